@@ -1,0 +1,158 @@
+/*
+ * kcg.h -- C-ABI of the MI355X (gfx950) kernels that stand in for the text the
+ * reference's CUDA emitter prints.
+ *
+ * The reference's backend entry is `std::string CUDAGen(mlir::ModuleOp&)`
+ * (include/Backend/CUDA.h:6, src/Backend/CUDA.cc:878-890).  It prints one
+ *     namespace <graph> { __global__ void kernelN(float* arg0, float* arg1, ...) }
+ * per optimised function (src/Backend/CUDA.cc:793-801), with raw device
+ * pointers in first-use order (A,B,C / Q,K,V,O), every size baked in, and the
+ * launch geometry only in a comment (src/Backend/CUDA.cc:786-791).  A harness
+ * outside the reference tree allocates, copies, launches and times
+ * (test/test.cc:27-34).  The entry points below are what such a harness binds
+ * instead: same operand order, caller-owned device pointers, row-major
+ * contiguous tensors, no hidden allocation, no implicit synchronisation; the
+ * launch is asynchronous on the given HIP stream (0 = the null stream).
+ *
+ * Unlike the reference (assert(false) / exit(EXIT_FAILURE), e.g.
+ * src/Frontend/Operators.cc:271, include/KernelCodeGen.h:78-81) nothing here
+ * aborts: every entry point returns a kcg_status.
+ *
+ * All entry points are thread-safe and hold no state between calls.
+ */
+#ifndef KCG_H
+#define KCG_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KCG_API __attribute__((visibility("default")))
+
+typedef enum kcg_status {
+  KCG_OK = 0,
+  KCG_ERR_NULL_POINTER = 1,      /* a required pointer argument is NULL        */
+  KCG_ERR_BAD_SHAPE = 2,         /* non-positive or overflowing extent         */
+  KCG_ERR_UNSUPPORTED_SHAPE = 3, /* extent not handled by the selected kernel  */
+  KCG_ERR_BAD_SCHEDULE = 4,      /* tile sizes that no kernel is built for     */
+  KCG_ERR_BAD_ARGUMENT = 5,      /* unknown epilogue / dtype / flag            */
+  KCG_ERR_LAUNCH = 6,            /* HIP reported an error at launch            */
+  KCG_ERR_NO_DEVICE = 7          /* no usable gfx950 device                    */
+} kcg_status;
+
+/* Human-readable text for a status (never NULL). */
+KCG_API const char *kcg_status_str(int status);
+
+/* Library version "major.minor.patch". */
+KCG_API const char *kcg_version(void);
+
+/* ---- tiled fp32 matmul (+ fused ReLU epilogue) ---------------------------- */
+
+/* Epilogue applied to each C element before it is stored.  KCG_EPILOGUE_RELU is
+ * arith.maxf(0, x) as the reference's Relu operator defines it
+ * (src/Frontend/Operators.cc:238-242): NaN propagates, -0 becomes +0.  The
+ * reference never fuses it (its emitter skips the Relu function,
+ * src/Backend/CUDA.cc:859-866); the fusion is an extension. */
+typedef enum kcg_epilogue { KCG_EPILOGUE_NONE = 0, KCG_EPILOGUE_RELU = 1 } kcg_epilogue;
+
+/* Schedule of the matmul kernel: the string-keyed tile table of the reference
+ * (include/KernelCodeGen.h:34-37: BLOCK_SIZE_M/N/K, GROUP_SIZE_M, THREAD_SIZE_M/N,
+ * VECTORIZE_WIDTH, WARP_SIZE) as a plain struct.  A NULL schedule, or a field
+ * set to 0, selects the built-in default for gfx950 (256 x 128 x 16 block tile,
+ * wave64, 64 x 64 per-wave tile of 32x32x2 fp32 MFMA blocks, group_m 8). */
+typedef struct kcg_gemm_sched {
+  int32_t block_m;   /* BLOCK_SIZE_M: rows of C per workgroup                  */
+  int32_t block_n;   /* BLOCK_SIZE_N: columns of C per workgroup               */
+  int32_t block_k;   /* BLOCK_SIZE_K: K-slice staged in LDS per step           */
+  int32_t group_m;   /* GROUP_SIZE_M: M-tiles per rasterisation group          */
+  int32_t wave_m;    /* rows of C per wavefront (the THREAD_SIZE_M analogue)   */
+  int32_t wave_n;    /* columns of C per wavefront (THREAD_SIZE_N analogue)    */
+  int32_t vec_width; /* VECTORIZE_WIDTH: floats per global/LDS access (4)      */
+  int32_t wave_size; /* WARP_SIZE: must be 64 (or 0) on gfx950                 */
+} kcg_gemm_sched;
+
+/* C[M,N] = epilogue(A[M,K] . B[K,N]); fp32, row-major, contiguous.
+ * Replaces `<graph>::kernel0(float* A, float* B, float* C)` as generated for
+ * Matmul_m<M>n<N>k<K> (src/Optimizer/Optimizer.cc:383-548; prototype
+ * src/Backend/CUDA.cc:793-801; adaptor contract test/test.cc:27-33).
+ * Any M, N, K >= 1 is accepted (the reference requires M, N % 128 == 0 and
+ * K % 8 == 0, src/Optimizer/Rewriter.cc:124-128); ragged edges take a
+ * bounds-checked path.  A, B, C must not alias. */
+KCG_API int kcg_gemm_f32(const float *A, const float *B, float *C, int64_t M,
+                         int64_t N, int64_t K, int epilogue,
+                         const kcg_gemm_sched *sched, void *stream);
+
+/* Launch geometry the call above would use, for logging in the reference's
+ * "// grid dims:(..), block dims:(..)" style (src/Backend/CUDA.cc:786-791). */
+typedef struct kcg_launch_info {
+  int32_t grid[3];
+  int32_t block[3];
+  int32_t lds_bytes;
+  int32_t waves_per_block;
+  char kernel[64];
+} kcg_launch_info;
+
+KCG_API int kcg_gemm_f32_query(int64_t M, int64_t N, int64_t K,
+                               const kcg_gemm_sched *sched, kcg_launch_info *out);
+
+/* ---- fused multi-head attention ------------------------------------------ */
+
+/* Schedule of the FMHA kernel: the reference's table (include/KernelCodeGen.h:
+ * 38-41; Br = HdxBr / Hd, Bc = BrxBc / Br, src/Optimizer/Optimizer.cc:1136-1144)
+ * reduced to the two tile extents.  NULL or 0 selects the gfx950 default. */
+typedef struct kcg_fmha_sched {
+  int32_t br; /* query rows per workgroup                                      */
+  int32_t bc; /* key/value rows per inner step                                 */
+} kcg_fmha_sched;
+
+/* O = softmax(scale * Q.K^T [+ causal mask]) . V, all [B,H,S,D] contiguous fp32.
+ * Replaces the kernel generated for
+ * Fused_Multi_Head_Attention_<b>_<h>_SL<S>_HD<D>(Q,K,V,O)
+ * (src/Optimizer/Optimizer.cc:1101-1118); semantics are those of the Frontend
+ * graph BatchedMatmul(Q,K^T) -> Softmax(axis -1) -> BatchedMatmul(P,V)
+ * (test/test.cc:88-90).  scale = 1 and causal = 0 give exactly that graph;
+ * scale and causal are extensions.  D must be 64 or 128; any S >= 1. */
+KCG_API int kcg_fmha_f32(const float *Q, const float *K, const float *V, float *O,
+                         int32_t B, int32_t H, int32_t S, int32_t D, float scale,
+                         int causal, const kcg_fmha_sched *sched, void *stream);
+
+typedef enum kcg_dtype { KCG_F32 = 0, KCG_BF16 = 1 } kcg_dtype;
+
+/* Same, with Q, K, V holding bf16 bit patterns (extension: the reference knows
+ * only float32/float64/float16, src/Frontend/Operators.cc:5-10).  Products are
+ * bf16 x bf16 accumulated in fp32; softmax in fp32; P is rounded to bf16 before
+ * the second product.  O is written as o_dtype (KCG_BF16 or KCG_F32). */
+KCG_API int kcg_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                          void *O, int o_dtype, int32_t B, int32_t H, int32_t S,
+                          int32_t D, float scale, int causal,
+                          const kcg_fmha_sched *sched, void *stream);
+
+KCG_API int kcg_fmha_query(int dtype, int32_t B, int32_t H, int32_t S, int32_t D,
+                           int causal, const kcg_fmha_sched *sched,
+                           kcg_launch_info *out);
+
+/* ---- un-fused operators (graphs the two patterns above do not match) ------ */
+
+/* y = maxf(0, x) elementwise; y may equal x (MemorySpace::inplace).
+ * src/Frontend/Operators.cc:182-250. */
+KCG_API int kcg_relu_f32(const float *x, float *y, int64_t n, void *stream);
+
+/* C[b] = op(A[b]) . op(B[b]) for `batch` contiguous matrices.
+ * transA = 0: A is [batch,M,K]; 1: [batch,K,M].  transB = 0: B is [batch,K,N];
+ * 1: [batch,N,K].  src/Frontend/Operators.cc:253-420 (name suffix _NN/_NT/...,
+ * :329-339). */
+KCG_API int kcg_batched_matmul_f32(const float *A, int transA, const float *B,
+                                   int transB, float *C, int64_t batch, int64_t M,
+                                   int64_t N, int64_t K, void *stream);
+
+/* In-place softmax over the last axis of a [rows, n] tensor:
+ * x = exp(x) / sum(exp(x)).  src/Frontend/Operators.cc:425-542. */
+KCG_API int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KCG_H */

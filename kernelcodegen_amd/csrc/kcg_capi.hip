@@ -1,0 +1,71 @@
+// Status strings, version, and the small un-fused elementwise operator.
+#include "kcg_common.h"
+
+namespace kcg {
+
+__global__ __launch_bounds__(256) void relu_f32_kernel(const float *__restrict__ x,
+                                                       float *__restrict__ y, int64_t n4,
+                                                       int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  for (; i < n4; i += stride) {
+    float4_t v = reinterpret_cast<const float4_t *>(x)[i];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = relu_maxf(v[e]);
+    reinterpret_cast<float4_t *>(y)[i] = v;
+  }
+  // tail (n % 4 elements), handled by the first threads of the grid
+  i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t t = n4 * 4 + i;
+  if (t < n) y[t] = relu_maxf(x[t]);
+}
+
+__global__ __launch_bounds__(256) void relu_f32_scalar_kernel(const float *__restrict__ x,
+                                                              float *__restrict__ y, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    y[i] = relu_maxf(x[i]);
+}
+
+}  // namespace kcg
+
+extern "C" {
+
+const char *kcg_status_str(int status) {
+  switch (status) {
+    case KCG_OK: return "ok";
+    case KCG_ERR_NULL_POINTER: return "null pointer argument";
+    case KCG_ERR_BAD_SHAPE: return "bad shape (non-positive or too large extent)";
+    case KCG_ERR_UNSUPPORTED_SHAPE: return "shape not supported by this kernel";
+    case KCG_ERR_BAD_SCHEDULE: return "no kernel is built for this schedule";
+    case KCG_ERR_BAD_ARGUMENT: return "bad argument (unknown epilogue, dtype or flag)";
+    case KCG_ERR_LAUNCH: return "HIP reported an error at kernel launch";
+    case KCG_ERR_NO_DEVICE: return "no usable gfx950 device";
+    default: return "unknown status";
+  }
+}
+
+const char *kcg_version(void) { return "0.1.0"; }
+
+int kcg_relu_f32(const float *x, float *y, int64_t n, void *stream) {
+  if (!x || !y) return KCG_ERR_NULL_POINTER;
+  if (n <= 0) return KCG_ERR_BAD_SHAPE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int threads = 256;
+  if (kcg::aligned16(x) && kcg::aligned16(y)) {
+    const int64_t n4 = n / 4;
+    int64_t blocks = (n4 + threads - 1) / threads;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    hipLaunchKernelGGL(kcg::relu_f32_kernel, dim3(static_cast<unsigned>(blocks)), dim3(threads), 0,
+                       s, x, y, n4, n);
+  } else {
+    int64_t blocks = (n + threads - 1) / threads;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    hipLaunchKernelGGL(kcg::relu_f32_scalar_kernel, dim3(static_cast<unsigned>(blocks)),
+                       dim3(threads), 0, s, x, y, n);
+  }
+  return kcg::launch_status();
+}
+
+}  // extern "C"
