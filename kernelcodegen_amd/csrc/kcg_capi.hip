@@ -47,6 +47,19 @@ const char *kcg_status_str(int status) {
 
 const char *kcg_version(void) { return "0.1.0"; }
 
+int kcg_fmha_query(int dtype, int32_t B, int32_t H, int32_t S, int32_t D, int causal,
+                   const kcg_fmha_sched *sched, kcg_launch_info *out) {
+  if (!out) return KCG_ERR_NULL_POINTER;
+  if (B <= 0 || H <= 0 || S <= 0 || D <= 0) return KCG_ERR_BAD_SHAPE;
+  if (dtype == KCG_F32)
+    return kcg::dispatch_fmha_f32(nullptr, nullptr, nullptr, nullptr, B, H, S, D, 1.0f, causal,
+                                  sched, nullptr, out);
+  if (dtype == KCG_BF16)
+    return kcg::dispatch_fmha_bf16(nullptr, nullptr, nullptr, nullptr, KCG_BF16, B, H, S, D, 1.0f,
+                                   causal, sched, nullptr, out);
+  return KCG_ERR_BAD_ARGUMENT;
+}
+
 int kcg_relu_f32(const float *x, float *y, int64_t n, void *stream) {
   if (!x || !y) return KCG_ERR_NULL_POINTER;
   if (n <= 0) return KCG_ERR_BAD_SHAPE;

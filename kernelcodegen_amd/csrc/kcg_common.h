@@ -39,6 +39,14 @@ inline int launch_status() {
   return hipGetLastError() == hipSuccess ? KCG_OK : KCG_ERR_LAUNCH;
 }
 
+// Defined in fmha_f32.hip / fmha_bf16.hip; `info` != nullptr only fills the launch geometry.
+int dispatch_fmha_f32(const float *Q, const float *K, const float *V, float *O, int B, int H, int S,
+                      int D, float scale, int causal, const kcg_fmha_sched *sched,
+                      hipStream_t stream, kcg_launch_info *info);
+int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O,
+                       int o_dtype, int B, int H, int S, int D, float scale, int causal,
+                       const kcg_fmha_sched *sched, hipStream_t stream, kcg_launch_info *info);
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace kcg

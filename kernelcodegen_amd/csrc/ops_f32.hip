@@ -1,0 +1,146 @@
+// Un-fused fp32 operators for graphs that neither the matmul nor the FMHA
+// pattern matches: BatchedMatmul (src/Frontend/Operators.cc:253-420) in its four
+// layout combinations, and the in-place last-axis Softmax (:425-542).
+#include "kcg_common.h"
+
+namespace kcg {
+
+// ---------------------------------------------------------------------------
+// Batched matmul: one 64x64 tile of C[b] per workgroup, 4 waves of one
+// v_mfma_f32_32x32x2_f32 block each, K walked in slices of 16 through LDS held
+// K-major ([k][m] and [k][n]) so both MFMA operands are read along M / N.
+// Loads are element-wise and bounds-checked, which makes every layout
+// ('N'/'T' for A and for B) and every extent legal.
+// ---------------------------------------------------------------------------
+template <bool TA, bool TB>
+__global__ __launch_bounds__(256) void bmm_f32_kernel(const float *__restrict__ A,
+                                                      const float *__restrict__ B,
+                                                      float *__restrict__ C, int M, int N, int K,
+                                                      int tiles_n) {
+  constexpr int BT = 64, BK = 16, PITCH = BT + 8;
+  __shared__ float As[BK * PITCH];
+  __shared__ float Bs[BK * PITCH];
+  const int64_t b = blockIdx.y;
+  const float *Ab = A + b * M * K;
+  const float *Bb = B + b * K * N;
+  float *Cb = C + b * M * N;
+  const int tile_m = blockIdx.x / tiles_n;
+  const int tile_n = blockIdx.x % tiles_n;
+  const int m0 = tile_m * BT, n0 = tile_n * BT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r32 = lane & 31, half = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  float16_t acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+
+  for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + i * 256;
+      // A: walk the contiguous global axis with the fastest thread index.
+      const int am = TA ? (idx % BT) : (idx / BK);
+      const int ak = TA ? (idx / BT) : (idx % BK);
+      const int gm = m0 + am, gk = k0 + ak;
+      float av = 0.0f;
+      if (gm < M && gk < K) av = TA ? Ab[static_cast<int64_t>(gk) * M + gm] : Ab[static_cast<int64_t>(gm) * K + gk];
+      As[ak * PITCH + am] = av;
+      const int bn = TB ? (idx / BK) : (idx % BT);
+      const int bk = TB ? (idx % BK) : (idx / BT);
+      const int gn = n0 + bn, gk2 = k0 + bk;
+      float bv = 0.0f;
+      if (gn < N && gk2 < K) bv = TB ? Bb[static_cast<int64_t>(gn) * K + gk2] : Bb[static_cast<int64_t>(gk2) * N + gn];
+      Bs[bk * PITCH + bn] = bv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      const float a = As[(kk + half) * PITCH + wm * 32 + r32];
+      const float bb = Bs[(kk + half) * PITCH + wn * 32 + r32];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bb, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  const int col = n0 + wn * 32 + r32;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int row = m0 + wm * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+    if (row < M && col < N) Cb[static_cast<int64_t>(row) * N + col] = acc[e];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Softmax over the last axis, in place, one workgroup per row.
+// x = exp(x - max) / sum(exp(x - max)): equal to the reference's
+// exp(x) / sum(exp(x)) by shift invariance, without its overflow for x > 88.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+__global__ __launch_bounds__(256) void softmax_f32_kernel(float *__restrict__ x, int64_t n) {
+  __shared__ float red[4];
+  float *row = x + static_cast<int64_t>(blockIdx.x) * n;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr float kLog2e = 1.4426950408889634f;
+
+  float m = -INFINITY;
+  for (int64_t i = tid; i < n; i += 256) m = fmaxf(m, row[i]);
+  m = wave_max(m);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  const float m_use = (m == -INFINITY) ? 0.0f : m;
+
+  float sum = 0.0f;
+  for (int64_t i = tid; i < n; i += 256) sum += exp2f((row[i] - m_use) * kLog2e);
+  sum = wave_sum(sum);
+  if (lane == 0) red[wave] = sum;
+  __syncthreads();
+  sum = (red[0] + red[1]) + (red[2] + red[3]);
+  const float inv = 1.0f / sum;
+  for (int64_t i = tid; i < n; i += 256) row[i] = exp2f((row[i] - m_use) * kLog2e) * inv;
+}
+
+}  // namespace kcg
+
+extern "C" {
+
+int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int transB, float *C,
+                           int64_t batch, int64_t M, int64_t N, int64_t K, void *stream) {
+  if (!A || !B || !C) return KCG_ERR_NULL_POINTER;
+  if (batch <= 0 || M <= 0 || N <= 0 || K <= 0) return KCG_ERR_BAD_SHAPE;
+  if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1)) return KCG_ERR_BAD_ARGUMENT;
+  const int64_t tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
+  if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL || tiles_m * tiles_n > 0x7fffffffLL ||
+      batch > 65535)
+    return KCG_ERR_BAD_SHAPE;
+  dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(batch));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
+  const int tn = static_cast<int>(tiles_n);
+  if (!transA && !transB) hipLaunchKernelGGL((kcg::bmm_f32_kernel<false, false>), grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
+  else if (!transA && transB) hipLaunchKernelGGL((kcg::bmm_f32_kernel<false, true>), grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
+  else if (transA && !transB) hipLaunchKernelGGL((kcg::bmm_f32_kernel<true, false>), grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
+  else hipLaunchKernelGGL((kcg::bmm_f32_kernel<true, true>), grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
+  return kcg::launch_status();
+}
+
+int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream) {
+  if (!x) return KCG_ERR_NULL_POINTER;
+  if (rows <= 0 || n <= 0 || rows > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL(kcg::softmax_f32_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), x, n);
+  return kcg::launch_status();
+}
+
+}  // extern "C"
