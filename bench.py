@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+A step is one launch of the fused fp32 matmul + ReLU kernel on BASELINE.json's
+configs[1] (M = N = K = 4096, A, B ~ N(0,1) from the seeded generator), inputs
+resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s, the roofline of the
+kernel (algorithmic FLOPs / HIP-event launch time vs the fp32 MFMA peak), the CPU
+oracle timed on the host cores, and the two attention workloads as extras.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (summaries under profiles/); None until measured.
+TRAFFIC_BYTES = {"gemm_cfg1": None, "fmha_cfg3": None, "fmha_cfg4": None}
+
+
+def time_launches(fn, steps, warmup):
+    """(wall ms per step, HIP-event ms per launch) over `steps` launches of fn."""
+    import torch
+    stream = torch.cuda.current_stream()
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)          # the kernels are launched on this same stream
+    for _ in range(steps):
+        fn()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the attention workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the matmul and attention kernels shard over row "
+                 "blocks / heads with no exchange step, and this build launches no multi-GPU run "
+                 "(use --gpus 1)")
+
+    import numpy as np
+    import torch
+    from kernelcodegen_amd import inputs, lib, ops
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    lib.load()
+    dev = torch.device("cuda:0")
+
+    # ---------------- headline: configs[1], fp32 4096^3 matmul + ReLU ----------------
+    cfg = inputs.config_inputs(1)
+    A_h, B_h = cfg["A"], cfg["B"]
+    M, K = A_h.shape
+    N = B_h.shape[1]
+    A = torch.from_numpy(A_h).to(dev)
+    B = torch.from_numpy(B_h).to(dev)
+    C = torch.empty((M, N), dtype=torch.float32, device=dev)
+    flops = 2.0 * M * N * K
+    alg_bytes = 4.0 * (M * K + K * N + M * N)
+    wall_ms, ev_ms = time_launches(lambda: ops.matmul(A, B, relu=True, out=C), args.steps, args.warmup)
+    value = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (ev_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "fp32 GEMM TFLOP/s + % FP32 peak; FMHA TFLOP/s at S=2048,d=128",
+        "value": round(value, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: fp32 matmul + fused ReLU, M=N=K=4096, row-major, "
+                               "A,B ~ N(0,1) seeded", "M": M, "N": N, "K": K, "epilogue": "relu"},
+        "pct_fp32_peak": round(100.0 * value / PEAK_FP32_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_TFLOPS, 4),
+                     "traffic": TRAFFIC_BYTES["gemm_cfg1"], "kernel": "gemm_f32_kernel",
+                     "algorithmic_flops": flops, "algorithmic_bytes": alg_bytes,
+                     "launch_ms": round(ev_ms, 5)},
+    }
+
+    # ---------------- CPU baseline: the oracle on the host cores ----------------
+    if not args.no_cpu:
+        from oracle import oracle
+        oracle.build()
+        dt = float("inf")
+        for _ in range(3):
+            t0 = time.perf_counter()
+            ref = oracle.relu(oracle.matmul(A_h, B_h))
+            dt = min(dt, time.perf_counter() - t0)
+        Ch = C.cpu().numpy()
+        d = np.abs(Ch.astype(np.float64) - ref)
+        rms = float(np.sqrt((ref.astype(np.float64) ** 2).mean()))
+        out["cpu_baseline"] = {
+            "value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.num_threads(),
+            "kind": "port", "sample": "the whole configs[1] workload (4096^3 matmul + ReLU), best of "
+                                      "3 runs, %.2f s wall each" % dt,
+            "gpu_vs_cpu_max_rel_err": float((d / np.maximum(np.abs(ref), rms)).max()),
+        }
+        del ref, Ch
+
+    # ---------------- extras: the two attention workloads ----------------
+    if not args.no_extras:
+        extras = {}
+        steps = max(5, args.steps // 2)
+        c3 = inputs.config_inputs(3)
+        Q, Kt, V = (torch.from_numpy(c3[k]).to(dev) for k in "QKV")
+        O = torch.empty_like(Q)
+        Bn, H, S, D = Q.shape
+        fl = 4.0 * Bn * H * S * S * D
+        w, e = time_launches(lambda: ops.fmha(Q, Kt, V, scale=c3["scale"], causal=False, out=O),
+                             steps, args.warmup)
+        extras["fmha_f32_cfg3"] = {
+            "workload": "configs[3]: fp32 FMHA B=1 H=32 S=2048 D=128 non-causal", "ms_per_step": round(w, 5),
+            "value": round(fl / (w * 1e-3) / 1e12, 3), "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(fl / (e * 1e-3) / 1e12, 3),
+                         "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(fl / (e * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4),
+                         "traffic": TRAFFIC_BYTES["fmha_cfg3"]}}
+        del Q, Kt, V, O
+        c4 = inputs.config_inputs(4)
+        Q, Kt, V = (torch.from_numpy(c4[k].view(np.int16)).to(dev).view(torch.bfloat16) for k in "QKV")
+        O = torch.empty_like(Q)
+        Bn, H, S, D = Q.shape
+        fl = 0.5 * 4.0 * Bn * H * S * S * D      # causal-counted (half of the full S^2 work)
+        w, e = time_launches(lambda: ops.fmha(Q, Kt, V, scale=c4["scale"], causal=True, out=O),
+                             steps, args.warmup)
+        extras["fmha_bf16_cfg4"] = {
+            "workload": "configs[4]: bf16 FMHA B=4 H=32 S=4096 D=128 causal, causal-counted FLOPs",
+            "ms_per_step": round(w, 5), "value": round(fl / (w * 1e-3) / 1e12, 3), "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(fl / (e * 1e-3) / 1e12, 3),
+                         "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(fl / (e * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+                         "traffic": TRAFFIC_BYTES["fmha_cfg4"]}}
+        out["extras"] = extras
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

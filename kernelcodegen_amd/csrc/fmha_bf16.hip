@@ -312,15 +312,9 @@ static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t
 #define KCG_LAUNCH(CAUSAL_, OBF_)                                                                 \
   do {                                                                                            \
     auto kern = fmha_bf16_kernel<D, BC, QT, CAUSAL_, OBF_>;                                       \
-    if (T::kLdsBytes > 48 * 1024) {                                                               \
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                               \
-                              hipFuncAttributeMaxDynamicSharedMemorySize,                         \
-                              T::kLdsBytes) != hipSuccess)                                        \
-        return KCG_ERR_LAUNCH;                                                                    \
-    }                                                                                             \
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads),              \
-                       T::kLdsBytes, stream, Q, K, V, O, S, static_cast<int>(q_blocks),           \
-                       scale_log2e);                                                              \
+    if (!allow_lds(kern, T::kLdsBytes)) return KCG_ERR_LAUNCH;                                    \
+    return launch(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads), T::kLdsBytes,     \
+                  stream, Q, K, V, O, S, static_cast<int>(q_blocks), scale_log2e);                \
   } while (0)
   const bool obf = o_dtype == KCG_BF16;
   if (causal) {
@@ -331,7 +325,6 @@ static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t
     else KCG_LAUNCH(false, false);
   }
 #undef KCG_LAUNCH
-  return launch_status();
 }
 
 int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O,

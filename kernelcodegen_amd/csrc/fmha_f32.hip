@@ -245,20 +245,13 @@ static int launch_fmha_f32(const float *Q, const float *K, const float *V, float
 #define KCG_LAUNCH(CAUSAL_)                                                                       \
   do {                                                                                            \
     auto kern = fmha_f32_kernel<D, BC, CAUSAL_>;                                                  \
-    if (T::kLdsBytes > 48 * 1024) {                                                               \
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                               \
-                              hipFuncAttributeMaxDynamicSharedMemorySize,                         \
-                              T::kLdsBytes) != hipSuccess)                                        \
-        return KCG_ERR_LAUNCH;                                                                    \
-    }                                                                                             \
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads),              \
-                       T::kLdsBytes, stream, Q, K, V, O, S, static_cast<int>(q_blocks),           \
-                       scale_log2e);                                                              \
+    if (!allow_lds(kern, T::kLdsBytes)) return KCG_ERR_LAUNCH;                                    \
+    return launch(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads), T::kLdsBytes,     \
+                  stream, Q, K, V, O, S, static_cast<int>(q_blocks), scale_log2e);                \
   } while (0)
   if (causal) KCG_LAUNCH(true);
   else KCG_LAUNCH(false);
 #undef KCG_LAUNCH
-  return launch_status();
 }
 
 int dispatch_fmha_f32(const float *Q, const float *K, const float *V, float *O, int B, int H, int S,

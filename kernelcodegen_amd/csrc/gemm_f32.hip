@@ -233,15 +233,10 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
 #define KCG_LAUNCH(RELU_, FULL_)                                                                 \
   do {                                                                                           \
     auto kern = gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N, RELU_, FULL_, MIN_WAVES>;          \
-    if (T::kLdsBytes > 48 * 1024) {                                                              \
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                              \
-                              hipFuncAttributeMaxDynamicSharedMemorySize,                        \
-                              T::kLdsBytes) != hipSuccess)                                       \
-        return KCG_ERR_LAUNCH;                                                                   \
-    }                                                                                            \
-    hipLaunchKernelGGL(kern, grid, block, T::kLdsBytes, stream, A, B, C, static_cast<int>(M),    \
-                       static_cast<int>(N), static_cast<int>(K), static_cast<int>(tiles_m),      \
-                       static_cast<int>(tiles_n), group_m);                                      \
+    if (!allow_lds(kern, T::kLdsBytes)) return KCG_ERR_LAUNCH;                                   \
+    return launch(kern, grid, block, T::kLdsBytes, stream, A, B, C, static_cast<int>(M),         \
+                  static_cast<int>(N), static_cast<int>(K), static_cast<int>(tiles_m),           \
+                  static_cast<int>(tiles_n), group_m);                                           \
   } while (0)
   if (relu) {
     if (full) KCG_LAUNCH(true, true);
@@ -251,7 +246,6 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
     else KCG_LAUNCH(false, false);
   }
 #undef KCG_LAUNCH
-  return launch_status();
 }
 
 // Resolves a schedule (NULL / zero fields = defaults) to one of the built tile

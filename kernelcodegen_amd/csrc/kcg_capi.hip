@@ -70,15 +70,14 @@ int kcg_relu_f32(const float *x, float *y, int64_t n, void *stream) {
     int64_t blocks = (n4 + threads - 1) / threads;
     if (blocks < 1) blocks = 1;
     if (blocks > 256 * 32) blocks = 256 * 32;
-    hipLaunchKernelGGL(kcg::relu_f32_kernel, dim3(static_cast<unsigned>(blocks)), dim3(threads), 0,
+    return kcg::launch(kcg::relu_f32_kernel, dim3(static_cast<unsigned>(blocks)), dim3(threads), 0,
                        s, x, y, n4, n);
   } else {
     int64_t blocks = (n + threads - 1) / threads;
     if (blocks > 256 * 32) blocks = 256 * 32;
-    hipLaunchKernelGGL(kcg::relu_f32_scalar_kernel, dim3(static_cast<unsigned>(blocks)),
+    return kcg::launch(kcg::relu_f32_scalar_kernel, dim3(static_cast<unsigned>(blocks)),
                        dim3(threads), 0, s, x, y, n);
   }
-  return kcg::launch_status();
 }
 
 }  // extern "C"

@@ -4,6 +4,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <utility>
+
 #include "kcg.h"
 
 namespace kcg {
@@ -35,8 +38,32 @@ __device__ __forceinline__ float relu_maxf(float x) {
   return (x > 0.0f || x != x) ? x : 0.0f;
 }
 
-inline int launch_status() {
-  return hipGetLastError() == hipSuccess ? KCG_OK : KCG_ERR_LAUNCH;
+// Launches `kern` and reports the launch's own status.  hipLaunchKernel returns
+// the error of this launch; hipGetLastError would also surface a stale error
+// left behind by an unrelated earlier runtime call of the host program.
+template <typename... KArgs, size_t... I>
+inline int launch_impl(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes,
+                       hipStream_t stream, std::tuple<KArgs...> &args, std::index_sequence<I...>) {
+  void *ptrs[] = {static_cast<void *>(&std::get<I>(args))...};
+  const hipError_t e =
+      hipLaunchKernel(reinterpret_cast<const void *>(kern), grid, block, ptrs, lds_bytes, stream);
+  return e == hipSuccess ? KCG_OK : KCG_ERR_LAUNCH;
+}
+
+template <typename... KArgs, typename... Args>
+inline int launch(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes,
+                  hipStream_t stream, Args... args) {
+  static_assert(sizeof...(KArgs) == sizeof...(Args), "kernel argument count");
+  std::tuple<KArgs...> packed{static_cast<KArgs>(args)...};
+  return launch_impl(kern, grid, block, lds_bytes, stream, packed, std::index_sequence_for<KArgs...>{});
+}
+
+// Kernels that need more than 48 KiB of dynamic LDS must opt in once per function.
+template <typename... KArgs>
+inline bool allow_lds(void (*kern)(KArgs...), int lds_bytes) {
+  if (lds_bytes <= 48 * 1024) return true;
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) == hipSuccess;
 }
 
 // Defined in fmha_f32.hip / fmha_bf16.hip; `info` != nullptr only fills the launch geometry.

@@ -128,19 +128,17 @@ int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int trans
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
   const int tn = static_cast<int>(tiles_n);
-  if (!transA && !transB) hipLaunchKernelGGL((kcg::bmm_f32_kernel<false, false>), grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
-  else if (!transA && transB) hipLaunchKernelGGL((kcg::bmm_f32_kernel<false, true>), grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
-  else if (transA && !transB) hipLaunchKernelGGL((kcg::bmm_f32_kernel<true, false>), grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
-  else hipLaunchKernelGGL((kcg::bmm_f32_kernel<true, true>), grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
-  return kcg::launch_status();
+  if (!transA && !transB) return kcg::launch(kcg::bmm_f32_kernel<false, false>, grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
+  if (!transA && transB) return kcg::launch(kcg::bmm_f32_kernel<false, true>, grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
+  if (transA && !transB) return kcg::launch(kcg::bmm_f32_kernel<true, false>, grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
+  return kcg::launch(kcg::bmm_f32_kernel<true, true>, grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
 }
 
 int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream) {
   if (!x) return KCG_ERR_NULL_POINTER;
   if (rows <= 0 || n <= 0 || rows > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL(kcg::softmax_f32_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0,
+  return kcg::launch(kcg::softmax_f32_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), x, n);
-  return kcg::launch_status();
 }
 
 }  // extern "C"

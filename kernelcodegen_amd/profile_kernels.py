@@ -1,0 +1,60 @@
+#!/usr/bin/env python3
+"""Runs one workload's kernel a few times, preceded by a plain device-to-device
+copy of known size, so that a profiler run over this script sees both:
+
+    rocprofv3 --kernel-trace --stats -d OUT -- python3 kernelcodegen_amd/profile_kernels.py --workload gemm_cfg1
+    rocprofv3 --pmc FETCH_SIZE -d OUT -- python3 kernelcodegen_amd/profile_kernels.py --workload gemm_cfg1
+    rocprofv3 --pmc WRITE_SIZE -d OUT -- python3 kernelcodegen_amd/profile_kernels.py --workload gemm_cfg1
+
+The copy (COPY_MIB MiB read + COPY_MIB MiB written per launch) calibrates the
+FETCH_SIZE / WRITE_SIZE counters: the factor is bytes-known / counter-read.
+"""
+import argparse
+import os
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+COPY_MIB = 256
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--workload", default="gemm_cfg1",
+                    choices=["gemm_cfg0", "gemm_cfg1", "gemm_cfg2", "fmha_cfg3", "fmha_cfg4"])
+    ap.add_argument("--iters", type=int, default=5)
+    args = ap.parse_args()
+
+    import numpy as np
+    import torch
+    from kernelcodegen_amd import inputs, ops
+
+    dev = torch.device("cuda:0")
+    src = torch.empty(COPY_MIB * (1 << 20) // 4, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    for _ in range(args.iters):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
+    kind, cfg = args.workload.split("_cfg")
+    c = inputs.config_inputs(int(cfg))
+    if kind == "gemm":
+        A = torch.from_numpy(c["A"]).to(dev)
+        B = torch.from_numpy(c["B"]).to(dev)
+        C = torch.empty((A.shape[0], B.shape[1]), dtype=torch.float32, device=dev)
+        fn = lambda: ops.matmul(A, B, relu=c["relu"], out=C)
+    else:
+        if c["dtype"] == "bf16":
+            Q, K, V = (torch.from_numpy(c[k].view(np.int16)).to(dev).view(torch.bfloat16) for k in "QKV")
+        else:
+            Q, K, V = (torch.from_numpy(c[k]).to(dev) for k in "QKV")
+        O = torch.empty_like(Q)
+        fn = lambda: ops.fmha(Q, K, V, scale=c["scale"], causal=c["causal"], out=O)
+    for _ in range(args.iters):
+        fn()
+    torch.cuda.synchronize()
+    print("done", args.workload, args.iters)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,93 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol that
+include/kcg.h declares, and rejects bad arguments before touching the device.
+No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from kernelcodegen_amd import lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "kcg.h")).read()
+    return sorted(set(re.findall(r"KCG_API[^;(]*?\b(kcg_\w+)\s*\(", text)))
+
+
+def test_header_declares_what_python_binds():
+    assert _declared_symbols() == sorted(lib.SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    L = ctypes.CDLL(lib.LIB_PATH)
+    for name in _declared_symbols():
+        assert hasattr(L, name), name
+
+
+def test_status_strings():
+    L = lib.load()
+    assert L.kcg_version().decode().count(".") == 2
+    seen = set()
+    for code in range(0, 8):
+        s = lib.status_str(code)
+        assert s and s != "unknown status"
+        seen.add(s)
+    assert len(seen) == 8
+    assert lib.status_str(99) == "unknown status"
+
+
+def test_argument_validation_returns_status_not_abort():
+    L = lib.load()
+    one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+    assert L.kcg_gemm_f32(None, one, one, 128, 128, 8, 0, None, None) == 1
+    assert L.kcg_gemm_f32(one, one, one, 0, 128, 8, 0, None, None) == 2
+    assert L.kcg_gemm_f32(one, one, one, 128, 128, 8, 7, None, None) == 5
+    bad = lib.GemmSched(block_m=96, block_n=128, block_k=8)
+    assert L.kcg_gemm_f32(one, one, one, 128, 128, 8, 0, ctypes.byref(bad), None) == 4
+    bad = lib.GemmSched(wave_size=32)
+    assert L.kcg_gemm_f32(one, one, one, 128, 128, 8, 0, ctypes.byref(bad), None) == 4
+    assert L.kcg_fmha_f32(one, one, None, one, 1, 1, 128, 128, 1.0, 0, None, None) == 1
+    assert L.kcg_fmha_f32(one, one, one, one, 1, 1, 0, 128, 1.0, 0, None, None) == 2
+    assert L.kcg_fmha_f32(one, one, one, one, 1, 1, 128, 96, 1.0, 0, None, None) == 3
+    assert L.kcg_fmha_f32(one, one, one, one, 1, 1, 128, 128, 1.0, 2, None, None) == 5
+    assert L.kcg_fmha_f32(one, one, one, one, 1, 1, 128, 128, float("nan"), 0, None, None) == 5
+    assert L.kcg_fmha_f32(ctypes.c_void_p(4), one, one, one, 1, 1, 128, 128, 1.0, 0, None, None) == 5
+    bad = lib.FmhaSched(br=64, bc=64)
+    assert L.kcg_fmha_f32(one, one, one, one, 1, 1, 128, 128, 1.0, 0, ctypes.byref(bad), None) == 4
+    assert L.kcg_fmha_bf16(one, one, one, one, 3, 1, 1, 128, 128, 1.0, 0, None, None) == 5
+    assert L.kcg_fmha_bf16(one, one, one, None, 1, 1, 1, 128, 128, 1.0, 0, None, None) == 1
+    assert L.kcg_relu_f32(None, one, 4, None) == 1
+    assert L.kcg_relu_f32(one, one, 0, None) == 2
+    assert L.kcg_batched_matmul_f32(one, 2, one, 0, one, 1, 4, 4, 4, None) == 5
+    assert L.kcg_batched_matmul_f32(one, 0, one, 0, one, 0, 4, 4, 4, None) == 2
+    assert L.kcg_softmax_f32(None, 4, 4, None) == 1
+    assert L.kcg_softmax_f32(one, 4, 0, None) == 2
+
+
+def test_launch_geometry_queries():
+    L = lib.load()
+    info = lib.LaunchInfo()
+    # the reference's demo shape, with its own 128 x 128 x 8 tile: grid (32,16) = 512 tiles
+    s = lib.GemmSched(block_m=128, block_n=128, block_k=8, wave_m=64, wave_n=64)
+    assert L.kcg_gemm_f32_query(4096, 2048, 1024, ctypes.byref(s), ctypes.byref(info)) == 0
+    assert info.grid[0] == 32 * 16 and info.block[0] == 256
+    assert info.lds_bytes == 2 * (128 * 12 + 8 * 136) * 4
+    assert L.kcg_gemm_f32_query(4096, 4096, 4096, None, ctypes.byref(info)) == 0
+    assert info.grid[0] * 256 * 128 == 4096 * 4096 and info.lds_bytes <= 160 * 1024
+    assert L.kcg_gemm_f32_query(100, 100, 100, None, None) == 1
+    assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 1, None, ctypes.byref(info)) == 0
+    assert info.grid[0] % (4 * 32) == 0 and info.block[0] == 256
+    assert L.kcg_fmha_query(0, 1, 32, 2048, 128, 0, None, ctypes.byref(info)) == 0
+    assert info.grid[0] == 32 * 2048 // 128
+    assert L.kcg_fmha_query(7, 1, 1, 128, 128, 0, None, ctypes.byref(info)) == 5
+    assert L.kcg_fmha_query(0, 1, 1, 128, 80, 0, None, ctypes.byref(info)) == 3
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "LIB_PATH", "/nonexistent/libkcg_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        lib.load()

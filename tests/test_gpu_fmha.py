@@ -1,0 +1,182 @@
+"""GPU parity of the fused attention kernels against the CPU oracle.
+
+Tolerances (BASELINE.json north_star): max relative error 1e-4 for fp32 and
+2e-2 for bf16 inputs, on both figures of conftest.rel_err.  The oracle is run
+with the row-max shift (stable=True), which tests/test_oracle.py shows equal to
+the reference's literal exp(x)/sum(exp(x)) form.
+"""
+import numpy as np
+import pytest
+
+from conftest import rel_err
+from kernelcodegen_amd import inputs
+
+pytestmark = pytest.mark.gpu
+TOL_F32 = 1e-4
+TOL_BF16 = 2e-2
+
+
+def _gpu(x, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+
+
+def _gpu_bf16(bits, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(dev).view(torch.bfloat16)
+
+
+SHAPES = [(1, 2, 128, 128), (1, 2, 256, 64), (2, 3, 200, 128), (1, 1, 77, 64), (1, 1, 1, 128),
+          (1, 2, 33, 64), (1, 2, 512, 128), (1, 1, 640, 64)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bc", [32, 64])
+def test_f32_parity(oracle, dev, shape, causal, bc):
+    from kernelcodegen_amd import ops
+    B, H, S, D = shape
+    Q, K, V = (inputs.normal(shape, 201, i) for i in range(3))
+    for scale in (D ** -0.5, 1.0 / 3):
+        ref = oracle.fmha(Q, K, V, scale=scale, causal=causal, stable=True)
+        O = ops.fmha(_gpu(Q, dev), _gpu(K, dev), _gpu(V, dev), scale=scale, causal=causal,
+                     sched=dict(br=128, bc=bc)).cpu().numpy()
+        assert max(rel_err(O, ref)) < TOL_F32
+
+
+def test_f32_reference_graph_scale_one(oracle, dev):
+    """scale = 1, no mask: the reference's own three-operator graph, literal softmax."""
+    from kernelcodegen_amd import ops
+    shape = (2, 2, 160, 64)
+    Q, K, V = (inputs.normal(shape, 202, i) for i in range(3))
+    Q = (Q * np.float32(0.25)).astype(np.float32)       # keep exp(x) in range for the literal form
+    ref = oracle.fmha(Q, K, V, scale=1.0, causal=False, stable=False)
+    graph = oracle.batched_matmul(oracle.softmax(oracle.batched_matmul(Q, 0, K, 1)), 0, V, 0)
+    assert np.array_equal(ref, graph)
+    O = ops.fmha(_gpu(Q, dev), _gpu(K, dev), _gpu(V, dev), scale=1.0, causal=False).cpu().numpy()
+    assert max(rel_err(O, ref)) < TOL_F32
+
+
+@pytest.mark.parametrize("shape", SHAPES + [(1, 1, 1024, 128)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("br", [128, 256])
+def test_bf16_parity(oracle, dev, shape, causal, br):
+    import torch
+    from kernelcodegen_amd import ops
+    B, H, S, D = shape
+    Q, K, V = (inputs.to_bf16_bits(inputs.normal(shape, 203, i)) for i in range(3))
+    scale = D ** -0.5
+    ref = oracle.fmha(Q, K, V, scale=scale, causal=causal, stable=True)
+    tq, tk, tv = (_gpu_bf16(t, dev) for t in (Q, K, V))
+    for odt in (torch.bfloat16, torch.float32):
+        O = ops.fmha(tq, tk, tv, scale=scale, causal=causal, out_dtype=odt,
+                     sched=dict(br=br, bc=64))
+        assert O.dtype == odt
+        assert max(rel_err(O.float().cpu().numpy(), ref)) < TOL_BF16
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_closed_forms(dev, dtype):
+    import torch
+    from kernelcodegen_amd import ops
+    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    tol = 1e-5 if dtype == "f32" else 1e-2
+    B, H, S, D = 1, 2, 300, 128
+    g = torch.Generator(device="cpu").manual_seed(5)
+    Q = torch.randn(B, H, S, D, generator=g).to(dev).to(tdt)
+    K = torch.randn(B, H, S, D, generator=g).to(dev).to(tdt)
+    V = torch.randn(B, H, S, D, generator=g).to(dev).to(tdt)
+    # V = 1 -> O = 1 (softmax rows sum to one)
+    for causal in (False, True):
+        O = ops.fmha(Q, K, torch.ones_like(V), scale=0.1, causal=causal, out_dtype=torch.float32)
+        assert float((O.float() - 1).abs().max()) < tol
+    # K = 0 -> uniform weights: mean of V, or prefix mean when causal
+    Z = torch.zeros_like(K)
+    O = ops.fmha(Q, Z, V, scale=1.0, causal=False, out_dtype=torch.float32).float()
+    mean = V.float().mean(2, keepdim=True).expand_as(O)
+    assert float((O - mean).abs().max()) < (1e-5 if dtype == "f32" else 3e-3)
+    Oc = ops.fmha(Q, Z, V, scale=1.0, causal=True, out_dtype=torch.float32).float()
+    prefix = V.float().cumsum(2) / torch.arange(1, S + 1, device=dev).view(1, 1, S, 1)
+    assert float((Oc - prefix).abs().max()) < (1e-5 if dtype == "f32" else 1.5e-2)
+    # causal: row 0 sees key 0 only
+    assert float((Oc[:, :, 0] - V.float()[:, :, 0]).abs().max()) < (1e-6 if dtype == "f32" else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_causal_future_keys_do_not_leak_and_heads_independent(dev, dtype):
+    import torch
+    from kernelcodegen_amd import ops
+    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    B, H, S, D = 2, 3, 257, 64
+    g = torch.Generator(device="cpu").manual_seed(6)
+    Q, K, V = (torch.randn(B, H, S, D, generator=g).to(dev).to(tdt) for _ in range(3))
+    O = ops.fmha(Q, K, V, scale=0.2, causal=True)
+    K2, V2 = K.clone(), V.clone()
+    K2[:, :, 130:] += 4
+    V2[:, :, 130:] -= 2
+    O2 = ops.fmha(Q, K2, V2, scale=0.2, causal=True)
+    assert torch.equal(O2[:, :, :130], O[:, :, :130])
+    assert not torch.equal(O2[:, :, 130:], O[:, :, 130:])
+    perm = torch.tensor([2, 0, 1], device=dev)
+    Op = ops.fmha(Q[:, perm].contiguous(), K[:, perm].contiguous(), V[:, perm].contiguous(),
+                  scale=0.2, causal=True)
+    assert torch.equal(Op, O[:, perm])
+
+
+def test_single_tile_vs_repeated_tiles(dev):
+    """Keys repeated 4x give the same softmax-weighted mean: exercises the
+    running max / sum / rescale across K/V tiles against the single-tile case."""
+    import torch
+    from kernelcodegen_amd import ops
+    g = torch.Generator(device="cpu").manual_seed(7)
+    Q = torch.randn(1, 2, 64, 128, generator=g).to(dev)
+    K = torch.randn(1, 2, 64, 128, generator=g).to(dev)
+    V = torch.randn(1, 2, 64, 128, generator=g).to(dev)
+    Qp = torch.cat([Q] * 4, 2).contiguous()
+    O1 = ops.fmha(Q, K, V, scale=0.1)
+    O4 = ops.fmha(Qp, torch.cat([K] * 4, 2).contiguous(), torch.cat([V] * 4, 2).contiguous(), scale=0.1)
+    assert float((O4[:, :, :64] - O1).abs().max()) < 1e-5
+
+
+def test_cfg3_full_size(oracle, dev):
+    """configs[3]: fp32, B=1 H=32 S=2048 D=128, non-causal; sampled query rows."""
+    from kernelcodegen_amd import ops
+    c = inputs.config_inputs(3)
+    O = ops.fmha(_gpu(c["Q"], dev), _gpu(c["K"], dev), _gpu(c["V"], dev), scale=c["scale"],
+                 causal=False).cpu().numpy()
+    for r0, r1 in [(0, 16), (1000, 1024), (2040, 2048)]:
+        ref = oracle.fmha(c["Q"], c["K"], c["V"], scale=c["scale"], causal=False, stable=True,
+                          rows=(r0, r1))
+        assert max(rel_err(O[:, :, r0:r1], ref)) < TOL_F32
+
+
+def test_cfg4_full_size(oracle, dev):
+    """configs[4]: bf16, B=4 H=32 S=4096 D=128, causal; sampled query rows and
+    the V = 1 property over the whole output."""
+    import torch
+    from kernelcodegen_amd import ops
+    c = inputs.config_inputs(4)
+    tq, tk, tv = (_gpu_bf16(c[k], dev) for k in "QKV")
+    for br in (128, 256):
+        O = ops.fmha(tq, tk, tv, scale=c["scale"], causal=True, sched=dict(br=br, bc=64))
+        Oh = O.float().cpu().numpy()
+        for r0, r1 in [(0, 8), (2043, 2051), (4088, 4096)]:
+            ref = oracle.fmha(c["Q"], c["K"], c["V"], scale=c["scale"], causal=True, stable=True,
+                              rows=(r0, r1))
+            assert max(rel_err(Oh[:, :, r0:r1], ref)) < TOL_BF16
+        ones = ops.fmha(tq, tk, torch.ones_like(tv), scale=c["scale"], causal=True,
+                        out_dtype=torch.float32, sched=dict(br=br, bc=64))
+        assert float((ones - 1).abs().max()) < 1e-2
+
+
+def test_errors(dev):
+    import torch
+    from kernelcodegen_amd import ops
+    from kernelcodegen_amd.lib import KcgError
+    q = torch.zeros(1, 1, 64, 96, device=dev)
+    with pytest.raises(KcgError) as e:
+        ops.fmha(q, q, q)
+    assert e.value.status == 3
+    q = torch.zeros(1, 1, 64, 64, device=dev)
+    with pytest.raises(ValueError):
+        ops.fmha(q, q[:, :, :32], q)

@@ -1,0 +1,160 @@
+"""GPU parity of the fp32 matmul (+ReLU) kernel against the CPU oracle.
+
+Tolerance: max relative error 1e-4 (fp32), as BASELINE.json's north_star states,
+on both error figures of conftest.rel_err.  The MFMA kernel sums the same
+products as the reference nest in a different order, so bit equality with the
+oracle is not expected; properties that the kernel's structure does fix
+bit-exactly (row permutation, ReLU of the un-fused result) are tested as such.
+"""
+import numpy as np
+import pytest
+
+from conftest import rel_err
+from kernelcodegen_amd import inputs
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+SCHEDS = [
+    None,
+    dict(block_m=128, block_n=128, block_k=8, wave_m=64, wave_n=64),    # the reference's tile
+    dict(block_m=128, block_n=128, block_k=16, wave_m=64, wave_n=64),
+    dict(block_m=128, block_n=128, block_k=32, wave_m=64, wave_n=64),
+    dict(block_m=256, block_n=128, block_k=32, wave_m=64, wave_n=64),
+    dict(block_m=256, block_n=256, block_k=16, wave_m=128, wave_n=128),
+    dict(block_m=64, block_n=64, block_k=32, wave_m=32, wave_n=32),
+]
+
+
+def _gpu(x, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 8), (256, 128, 16), (384, 256, 96), (512, 512, 512)])
+@pytest.mark.parametrize("sched", SCHEDS)
+def test_tile_aligned_shapes(oracle, dev, shape, sched):
+    from kernelcodegen_amd import ops
+    M, N, K = shape
+    A = inputs.uniform((M, K), 101, 0)
+    B = inputs.uniform((K, N), 101, 1)
+    ref = oracle.matmul(A, B)
+    C = ops.matmul(_gpu(A, dev), _gpu(B, dev), sched=sched).cpu().numpy()
+    assert max(rel_err(C, ref)) < TOL
+    Cr = ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=True, sched=sched).cpu().numpy()
+    assert np.array_equal(Cr, oracle.relu(C))          # fused epilogue == ReLU of the plain result
+    assert max(rel_err(Cr, oracle.relu(ref))) < TOL
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 3, 2), (131, 77, 19), (200, 136, 52), (129, 257, 33),
+                                   (300, 128, 7), (64, 1000, 130)])
+@pytest.mark.parametrize("sched", [None, SCHEDS[1], SCHEDS[6]])
+def test_ragged_shapes(oracle, dev, shape, sched):
+    from kernelcodegen_amd import ops
+    M, N, K = shape
+    A = inputs.normal((M, K), 102, 0)
+    B = inputs.normal((K, N), 102, 1)
+    C = ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=True, sched=sched).cpu().numpy()
+    assert C.shape == (M, N)
+    assert max(rel_err(C, oracle.relu(oracle.matmul(A, B)))) < TOL
+
+
+def test_exact_closed_forms(dev):
+    import torch
+    from kernelcodegen_amd import ops
+    n = 256
+    rng = np.random.default_rng(0)
+    A = rng.standard_normal((n, n)).astype(np.float32)
+    eye = torch.eye(n, device=dev)
+    assert np.array_equal(ops.matmul(_gpu(A, dev), eye).cpu().numpy(), A)
+    assert np.array_equal(ops.matmul(eye, _gpu(A, dev)).cpu().numpy(), A)
+    C = ops.matmul(torch.ones(128, 4096, device=dev), torch.ones(4096, 128, device=dev))
+    assert bool((C == 4096).all())
+    Ai = rng.integers(-8, 9, (256, 512)).astype(np.float32)
+    Bi = rng.integers(-8, 9, (512, 384)).astype(np.float32)
+    expect = (Ai.astype(np.int64) @ Bi.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(ops.matmul(_gpu(Ai, dev), _gpu(Bi, dev)).cpu().numpy(), expect)
+    # tile / lane mapping: A[i,k] = i, B = first row of ones -> C[i,j] = i
+    Am = np.repeat(np.arange(512, dtype=np.float32)[:, None], 64, axis=1)
+    Bm = np.zeros((64, 256), np.float32)
+    Bm[0] = 1
+    got = ops.matmul(_gpu(Am, dev), _gpu(Bm, dev)).cpu().numpy()
+    assert np.array_equal(got, np.repeat(np.arange(512, dtype=np.float32)[:, None], 256, axis=1))
+
+
+def test_relu_epilogue_special_values(dev):
+    import torch
+    from kernelcodegen_amd import ops
+    # diag(x) . I reproduces x on the diagonal exactly; everything else is +0
+    x = torch.tensor([-3.0, -0.0, 0.0, 2.5, float("-inf"), float("inf"), float("nan"), 1e-30],
+                     device=dev)
+    n = 128
+    A = torch.zeros(n, n, device=dev)
+    A[:8, :8] = torch.diag(x)
+    A[4, 4] = 0
+    A[5, 5] = 0
+    A[6, 6] = 0          # keep inf/nan out of the products that feed other elements
+    A[4, 9] = float("-inf")
+    A[5, 10] = float("inf")
+    A[6, 11] = float("nan")
+    B = torch.eye(n, device=dev)
+    C = ops.matmul(A, B, relu=True).cpu().numpy()
+    assert C[0, 0] == 0 and C[3, 3] == 2.5 and C[7, 7] == np.float32(1e-30)
+    assert C[1, 1] == 0 and not np.signbit(C[1, 1])
+    assert C[4, 9] == 0 and C[5, 10] == np.inf and np.isnan(C[6, 11])
+
+
+def test_row_permutation_is_bit_exact(dev):
+    import torch
+    from kernelcodegen_amd import ops
+    g = torch.Generator(device="cpu").manual_seed(3)
+    A = torch.randn(1024, 768, generator=g).to(dev)
+    B = torch.randn(768, 512, generator=g).to(dev)
+    perm = torch.randperm(1024, generator=g).to(dev)
+    C = ops.matmul(A, B)
+    Cp = ops.matmul(A[perm].contiguous(), B)
+    assert torch.equal(Cp, C[perm])
+
+
+def test_group_m_does_not_change_results(dev):
+    import torch
+    from kernelcodegen_amd import ops
+    A = torch.randn(1024, 256, device=dev)
+    B = torch.randn(256, 1536, device=dev)
+    ref = ops.matmul(A, B)
+    for g in (1, 3, 8, 64):
+        assert torch.equal(ops.matmul(A, B, sched=dict(group_m=g)), ref)
+
+
+@pytest.mark.parametrize("cfg", [0, 1, 2])
+def test_baseline_configs_full_size(oracle, dev, cfg):
+    """configs[0..2] at full size: sampled row bands against the oracle, plus
+    linearity in A (exact scaling by 2) over the whole output."""
+    import torch
+    from kernelcodegen_amd import ops
+    c = inputs.config_inputs(cfg)
+    A, B, relu = c["A"], c["B"], c["relu"]
+    M = A.shape[0]
+    dA, dB = _gpu(A, dev), _gpu(B, dev)
+    C = ops.matmul(dA, dB, relu=relu)
+    # scaling A by 2 is exact in fp32, so the result must scale exactly
+    C2 = ops.matmul(dA * 2, dB, relu=relu)
+    assert torch.equal(C2, C * 2)
+    Ch = C.cpu().numpy()
+    bands = [(0, 64), (M // 2 - 37, M // 2 + 27), (M - 64, M)]
+    for r0, r1 in bands:
+        ref = oracle.matmul_rows(A, B, r0, r1)
+        if relu:
+            ref = oracle.relu(ref)
+        assert max(rel_err(Ch[r0:r1], ref)) < TOL
+
+
+def test_shape_mismatch_raises(dev):
+    import torch
+    from kernelcodegen_amd import ops
+    with pytest.raises(ValueError, match="K-dim"):
+        ops.matmul(torch.zeros(4, 5, device=dev), torch.zeros(6, 4, device=dev))
+    from kernelcodegen_amd.lib import KcgError
+    with pytest.raises(KcgError):
+        ops.matmul(torch.zeros(128, 8, device=dev), torch.zeros(8, 128, device=dev),
+                   sched=dict(block_m=96))
