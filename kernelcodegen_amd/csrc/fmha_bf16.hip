@@ -72,7 +72,10 @@ __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
   uint16_t *Ks = lds16;
   uint16_t *Vs = lds16 + BC * T::kPitchK;
 
-  const int bid = blockIdx.x;
+  // Every XCD walks a contiguous range of (head, query block) ids, head-major, so
+  // the K/V of a head are fetched into one XCD's L2 only; heavy (late) query
+  // blocks first when causal.
+  const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qb_raw = bid % q_blocks;
   const int bh = bid / q_blocks;
   const int qb = CAUSAL ? (q_blocks - 1 - qb_raw) : qb_raw;

@@ -53,8 +53,10 @@ __global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restric
   float *Ks = lds;
   float *Vs = lds + BC * T::kPitchK;
 
-  // Heavy (late) query blocks first when causal, so the tail of the grid is cheap.
-  const int bid = blockIdx.x;
+  // Every XCD walks a contiguous range of (head, query block) ids, head-major, so
+  // the K/V of a head are fetched into one XCD's L2 only.  Heavy (late) query
+  // blocks first when causal, so the tail of the grid is cheap.
+  const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int bh = bid / q_blocks;
   const int qb_raw = bid - bh * q_blocks;
   const int qb = CAUSAL ? (q_blocks - 1 - qb_raw) : qb_raw;

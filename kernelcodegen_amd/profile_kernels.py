@@ -22,7 +22,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="gemm_cfg1",
                     choices=["gemm_cfg0", "gemm_cfg1", "gemm_cfg2", "fmha_cfg3", "fmha_cfg4"])
-    ap.add_argument("--iters", type=int, default=5)
+    ap.add_argument("--iters", type=int, default=40)
     args = ap.parse_args()
 
     import numpy as np
