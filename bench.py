@@ -21,9 +21,10 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (summaries under profiles/); None until measured.
-TRAFFIC_BYTES = {"gemm_cfg1": None, "fmha_cfg3": None, "fmha_cfg4": None}
+# HBM bytes per launch (fetch + write) measured with rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE, each scaled by the same counter's reading for a 256 MiB copy
+# (profiles/gemm_f32_cfg1.md, profiles/fmha_f32_cfg3.md, profiles/fmha_bf16_cfg4.md).
+TRAFFIC_BYTES = {"gemm_cfg1": 912872482, "fmha_cfg3": 134350917, "fmha_cfg4": 540614545}
 
 
 def time_launches(fn, steps, warmup):
