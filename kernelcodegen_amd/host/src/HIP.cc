@@ -1,0 +1,174 @@
+#include "Backend/HIP.h"
+
+#include <cstdio>
+#include <iostream>
+#include <sstream>
+
+#include "Optimizer/Analyzer.h"
+
+namespace KernelCodeGen {
+
+using namespace ir;
+
+namespace {
+
+int attrInt(FuncOp f, const std::string &key, int fallback) {
+  const std::string v = f.getAttr(key);
+  return v.empty() ? fallback : std::stoi(v);
+}
+
+bool bindMatmul(FuncOp f, KernelBinding &b) {
+  auto args = f.getArguments();
+  if (args.size() != 3) return false;
+  const auto &ta = args[0].getMemRefType();
+  const auto &tb = args[1].getMemRefType();
+  if (ta.elem != DType::f32 || tb.elem != DType::f32 || ta.shape.size() != 2 || tb.shape.size() != 2) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": only float32 rank-2 matmul has a gfx950 kernel\n";
+    return false;
+  }
+  b.kind = KernelBinding::Gemm;
+  b.entry = "kcg_gemm_f32";
+  b.M = ta.shape[0];
+  b.K = ta.shape[1];
+  b.N = tb.shape[1];
+  b.epilogue = f.getAttr("kcg.epilogue") == "relu" ? KCG_EPILOGUE_RELU : KCG_EPILOGUE_NONE;
+  b.gemmSched.block_m = attrInt(f, "kcg.BLOCK_SIZE_M", 0);
+  b.gemmSched.block_n = attrInt(f, "kcg.BLOCK_SIZE_N", 0);
+  b.gemmSched.block_k = attrInt(f, "kcg.BLOCK_SIZE_K", 0);
+  b.gemmSched.group_m = attrInt(f, "kcg.GROUP_SIZE_M", 0);
+  b.gemmSched.wave_m = attrInt(f, "kcg.WAVE_SIZE_M", 0);
+  b.gemmSched.wave_n = attrInt(f, "kcg.WAVE_SIZE_N", 0);
+  b.gemmSched.vec_width = attrInt(f, "kcg.VECTORIZE_WIDTH", 0);
+  b.gemmSched.wave_size = attrInt(f, "kcg.WARP_SIZE", 0);
+  b.argNames = {"A", "B", "C"};
+  const int st = kcg_gemm_f32_query(b.M, b.N, b.K, &b.gemmSched, &b.launch);
+  if (st != KCG_OK) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": " << kcg_status_str(st) << "\n";
+    return false;
+  }
+  return true;
+}
+
+bool bindFmha(FuncOp f, KernelBinding &b) {
+  auto args = f.getArguments();
+  if (args.size() != 4) return false;
+  const auto &tq = args[0].getMemRefType();
+  if (tq.shape.size() < 3) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": attention needs [batch.., S, D] operands\n";
+    return false;
+  }
+  const size_t r = tq.shape.size();
+  int64_t batch = 1;
+  for (size_t d = 0; d + 3 < r; ++d) batch *= tq.shape[d];
+  b.kind = KernelBinding::Fmha;
+  b.B = static_cast<int>(r >= 4 ? batch : 1);
+  b.H = static_cast<int>(tq.shape[r - 3]);
+  b.S = static_cast<int>(tq.shape[r - 2]);
+  b.D = static_cast<int>(tq.shape[r - 1]);
+  if (tq.elem == DType::f32) {
+    b.dtype = KCG_F32;
+    b.entry = "kcg_fmha_f32";
+  } else if (tq.elem == DType::bf16) {
+    b.dtype = KCG_BF16;
+    b.entry = "kcg_fmha_bf16";
+  } else {
+    std::cerr << "HIPBind: " << f.getSymName() << ": only float32 and bfloat16 attention kernels exist\n";
+    return false;
+  }
+  b.fmhaSched.br = attrInt(f, "kcg.Br", 0);
+  b.fmhaSched.bc = attrInt(f, "kcg.Bc", 0);
+  const std::string sc = f.getAttr("kcg.scale");
+  b.scale = sc.empty() ? 1.0f : std::stof(sc);
+  b.causal = attrInt(f, "kcg.causal", 0);
+  b.argNames = {"Q", "K", "V", "O"};
+  const int st = kcg_fmha_query(b.dtype, b.B, b.H, b.S, b.D, b.causal, &b.fmhaSched, &b.launch);
+  if (st != KCG_OK) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": " << kcg_status_str(st) << "\n";
+    return false;
+  }
+  return true;
+}
+
+}  // namespace
+
+std::vector<KernelBinding> HIPBind(ModuleOp &module) {
+  std::vector<KernelBinding> out;
+  // module order of the calls decides kernel numbering, as the emitter numbers kernels in walk order
+  for (auto call : Analyzer::collectFuncCalls(module)) {
+    FuncOp f = Analyzer::getTargetFunction(module, call.getCallee());
+    if (!f || f.getAttr("func.state") != "gpu") continue;
+    KernelBinding b;
+    b.graph = module.getName();
+    b.funcName = f.getSymName();
+    bool ok = false;
+    if (b.funcName.rfind("Matmul_m", 0) == 0) ok = bindMatmul(f, b);
+    else if (b.funcName.rfind("Fused_Multi_Head_Attention", 0) == 0) ok = bindFmha(f, b);
+    else std::cerr << "HIPBind: no gfx950 kernel is bound to " << b.funcName << "\n";
+    if (!ok) continue;
+    b.index = static_cast<int>(out.size());
+    out.push_back(b);
+  }
+  return out;
+}
+
+std::string HIPGen(ModuleOp &module) {
+  std::ostringstream os;
+  auto bindings = HIPBind(module);
+  os << "// Launchers for graph \"" << module.getName() << "\": each kernelN forwards to a prebuilt\n"
+     << "// gfx950 kernel of libkcg_hip.so (include/kcg.h).  Arguments are device pointers;\n"
+     << "// the call is asynchronous on `stream` and returns a kcg_status.\n"
+     << "#include \"kcg.h\"\n\n"
+     << "namespace " << module.getName() << " {\n\n";
+  for (auto &b : bindings) {
+    os << "// " << b.funcName << " -> " << b.launch.kernel << "\n"
+       << "// grid dims:(" << b.launch.grid[0] << ", " << b.launch.grid[1] << ", " << b.launch.grid[2]
+       << "), block dims:(" << b.launch.block[0] << ", " << b.launch.block[1] << ", " << b.launch.block[2]
+       << "), lds bytes:" << b.launch.lds_bytes << "\n";
+    if (b.kind == KernelBinding::Gemm) {
+      os << "inline int kernel" << b.index
+         << "(const float* arg0 /*A*/, const float* arg1 /*B*/, float* arg2 /*C*/, void* stream = nullptr) {\n"
+         << "  static const kcg_gemm_sched sched = {" << b.gemmSched.block_m << ", " << b.gemmSched.block_n << ", "
+         << b.gemmSched.block_k << ", " << b.gemmSched.group_m << ", " << b.gemmSched.wave_m << ", "
+         << b.gemmSched.wave_n << ", " << b.gemmSched.vec_width << ", " << b.gemmSched.wave_size << "};\n"
+         << "  return kcg_gemm_f32(arg0, arg1, arg2, " << b.M << ", " << b.N << ", " << b.K << ", "
+         << (b.epilogue == KCG_EPILOGUE_RELU ? "KCG_EPILOGUE_RELU" : "KCG_EPILOGUE_NONE") << ", &sched, stream);\n"
+         << "}\n\n";
+    } else {
+      char sc[64];
+      snprintf(sc, sizeof sc, "%.9gf", static_cast<double>(b.scale));
+      std::string scale = sc;
+      if (scale.find('.') == std::string::npos && scale.find('e') == std::string::npos)
+        scale.insert(scale.size() - 1, ".0");
+      const bool bf = b.dtype == KCG_BF16;
+      const char *ct = bf ? "const uint16_t*" : "const float*";
+      os << "inline int kernel" << b.index << "(" << ct << " arg0 /*Q*/, " << ct << " arg1 /*K*/, " << ct
+         << " arg2 /*V*/, " << (bf ? "uint16_t*" : "float*") << " arg3 /*O*/, void* stream = nullptr) {\n"
+         << "  static const kcg_fmha_sched sched = {" << b.fmhaSched.br << ", " << b.fmhaSched.bc << "};\n";
+      if (bf)
+        os << "  return kcg_fmha_bf16(arg0, arg1, arg2, arg3, KCG_BF16, " << b.B << ", " << b.H << ", " << b.S
+           << ", " << b.D << ", " << scale << ", " << b.causal << ", &sched, stream);\n";
+      else
+        os << "  return kcg_fmha_f32(arg0, arg1, arg2, arg3, " << b.B << ", " << b.H << ", " << b.S << ", " << b.D
+           << ", " << scale << ", " << b.causal << ", &sched, stream);\n";
+      os << "}\n\n";
+    }
+  }
+  os << "}  // namespace " << module.getName() << "\n";
+  return os.str();
+}
+
+int HIPLaunch(const KernelBinding &b, const std::vector<void *> &p, void *stream) {
+  if (p.size() != b.argNames.size()) return KCG_ERR_BAD_ARGUMENT;
+  if (b.kind == KernelBinding::Gemm)
+    return kcg_gemm_f32(static_cast<const float *>(p[0]), static_cast<const float *>(p[1]),
+                        static_cast<float *>(p[2]), b.M, b.N, b.K, b.epilogue, &b.gemmSched, stream);
+  if (b.dtype == KCG_BF16)
+    return kcg_fmha_bf16(static_cast<const uint16_t *>(p[0]), static_cast<const uint16_t *>(p[1]),
+                         static_cast<const uint16_t *>(p[2]), p[3], KCG_BF16, b.B, b.H, b.S, b.D, b.scale,
+                         b.causal, &b.fmhaSched, stream);
+  return kcg_fmha_f32(static_cast<const float *>(p[0]), static_cast<const float *>(p[1]),
+                      static_cast<const float *>(p[2]), static_cast<float *>(p[3]), b.B, b.H, b.S, b.D, b.scale,
+                      b.causal, &b.fmhaSched, stream);
+}
+
+}  // namespace KernelCodeGen

@@ -1,0 +1,308 @@
+#include "Optimizer/Optimizer.h"
+
+#include <cstdio>
+#include <iostream>
+
+void BatchMatmulDescriptor::log() const {
+  std::cerr << "m = " << m << " n = " << n << " k = " << k << "\nbatch = ";
+  for (auto b : batch) std::cerr << b << ",";
+  std::cerr << "\ntrans A = " << transA << " transB = " << transB << "\n";
+}
+
+namespace KernelCodeGen {
+
+using namespace ir;
+
+std::map<std::string, int> MatmulOptimizer::matmulConfig;
+std::map<std::string, int> FMHAOptimizer::fmhaConfig;
+float FMHAOptimizer::scale = 1.0f;
+bool FMHAOptimizer::causal = false;
+
+#define DUMP(module)                                 \
+  do {                                               \
+    if (KCGLog::level == Log::Debug) (module).dump(); \
+  } while (0)
+
+bool identifyBatchMatmul(const std::string &name, BatchMatmulDescriptor &matmul) {
+  std::vector<std::string> frags;
+  std::string cur;
+  for (char c : name) {
+    if (c == '_') {
+      frags.push_back(cur);
+      cur.clear();
+    } else {
+      cur += c;
+    }
+  }
+  frags.push_back(cur);
+  // BatchMatmul, batch..., m<M>, n<N>, k<K>, <N|T><N|T>
+  if (frags.size() < 5 || frags[0] != "BatchMatmul") return false;
+  const std::string &lay = frags.back();
+  if (lay.size() != 2 || (lay[0] != 'N' && lay[0] != 'T') || (lay[1] != 'N' && lay[1] != 'T')) return false;
+  auto number = [](const std::string &s, size_t from, int &out) {
+    if (s.size() <= from) return false;
+    for (size_t i = from; i < s.size(); ++i)
+      if (s[i] < '0' || s[i] > '9') return false;
+    out = std::stoi(s.substr(from));
+    return true;
+  };
+  const size_t n = frags.size();
+  if (frags[n - 4][0] != 'm' || frags[n - 3][0] != 'n' || frags[n - 2][0] != 'k') return false;
+  if (!number(frags[n - 4], 1, matmul.m) || !number(frags[n - 3], 1, matmul.n) || !number(frags[n - 2], 1, matmul.k))
+    return false;
+  matmul.batch.clear();
+  for (size_t i = 1; i + 4 < n; ++i) {
+    int b = 0;
+    if (!number(frags[i], 0, b)) return false;
+    matmul.batch.push_back(b);
+  }
+  matmul.transA = lay[0] == 'T';
+  matmul.transB = lay[1] == 'T';
+  return true;
+}
+
+// ----------------------------------------------------------------- Matmul
+bool MatmulOptimizer::applicable(ModuleOp &module) {
+  clear();
+  for (auto &func : Analyzer::collectFunctions(module, "Matmul")) {
+    // "BatchMatmul_..." also contains "Matmul": only the plain operator is handled here
+    if (func.getSymName().rfind("Matmul_m", 0) != 0) continue;
+    if (func.getAttr("func.state") != "cpu") continue;
+    auto loops = Analyzer::collectFuncLoops(func);
+    auto args = func.getArguments();
+    if (loops.size() != 3 || args.size() != 3) continue;
+    if (matmuls.count(func)) std::cerr << "Duplicated Matmul in module\n";
+    matmuls.insert(func);
+    matmulLoops[func] = loops;
+    matmulBuffers[func] = MemoryBuffer{args[0], args[1], args[2]};
+  }
+  return !matmuls.empty();
+}
+
+void MatmulOptimizer::applyOptimzer(ModuleOp &module) {
+  auto cfg = [&](const char *key, int fallback) {
+    auto it = matmulConfig.find(key);
+    return it == matmulConfig.end() ? fallback : it->second;
+  };
+  for (auto matmul : matmuls) {
+    auto loops = matmulLoops[matmul];
+    ForOp loopM = loops[0], loopN = loops[1], loopK = loops[2];
+    const int bm = cfg("BLOCK_SIZE_M", 128), bn = cfg("BLOCK_SIZE_N", 128), bk = cfg("BLOCK_SIZE_K", 8);
+    const int tm = cfg("THREAD_SIZE_M", 8), tn = cfg("THREAD_SIZE_N", 8);
+    if (loopM.getUpperBound() % bm || loopN.getUpperBound() % bn || loopK.getUpperBound() % bk || bm % tm ||
+        bn % tn) {
+      // ragged shapes keep the naive nest; the backend binds the bounds-checked kernel
+      matmul.setAttr("func.state", "gpu");
+      matmul.setAttr("kcg.schedule", "edge");
+      continue;
+    }
+    matmul.setAttr("func.state", "gpu");
+
+    auto m_axes = Rewriter::split(loopM, 3, {tm, bm});
+    auto n_axes = Rewriter::split(loopN, 3, {tn, bn});
+    DUMP(module);
+    ForOp m_outer = m_axes[0], m_mider = m_axes[1], m_inner = m_axes[2];
+    ForOp n_outer = n_axes[0], n_mider = n_axes[1], n_inner = n_axes[2];
+
+    Rewriter::reorder({m_outer, n_outer, m_mider, n_mider, m_inner, n_inner});
+    DUMP(module);
+
+    auto gridLevel = Rewriter::parallel({m_outer, n_outer});
+    auto blockLevel = Rewriter::parallel({m_mider, n_mider});
+    DUMP(module);
+
+    std::vector<ForOp> kmn_axes{loopK, m_inner, n_inner};
+    Rewriter::bufferizeLoopCarryVar(kmn_axes);  // tileC: THREAD_SIZE_M x THREAD_SIZE_N registers
+    DUMP(module);
+
+    Rewriter::reorder({loopK, m_inner, n_inner});
+    DUMP(module);
+
+    Rewriter::split(loopK, 2, {bk});
+    DUMP(module);
+
+    Rewriter::unrollAttribute(module, 8);
+
+    int64_t blockThreads = 0, gridBlocks = 0;
+    Analyzer::getParallelNumber(blockLevel, blockThreads);
+    Analyzer::getParallelNumber(gridLevel, gridBlocks);
+    matmul.setAttr("kcg.schedule", "tiled");
+    matmul.setAttr("kcg.block_threads", std::to_string(blockThreads));
+    matmul.setAttr("kcg.grid_blocks", std::to_string(gridBlocks));
+  }
+
+  // Fold an in-place Relu on the matmul result into the kernel epilogue.
+  std::set<Op *> erased;
+  for (auto call : Analyzer::collectFuncCalls(module)) {
+    if (erased.count(call.op)) continue;
+    FuncOp callee = Analyzer::getTargetFunction(module, call.getCallee());
+    if (!callee || !matmuls.count(callee)) continue;
+    auto users = Analyzer::getUsers(module, call.getResult(0));
+    if (users.size() != 1 || users[0]->kind != OpKind::Call) continue;
+    CallOp reluCall(users[0]);
+    if (reluCall.getCallee().rfind("Relu_Elementwise", 0) != 0) continue;
+    FuncOp relu = Analyzer::getTargetFunction(module, reluCall.getCallee());
+    // in place: the Relu function returns its own argument
+    Op *ret = relu ? relu->lastOp() : nullptr;
+    if (!ret || ret->operands.empty() || ret->operands[0] != relu.getArguments()[0]) continue;
+    // only if no other matmul call shares the function with a different epilogue
+    callee.setAttr("kcg.epilogue", "relu");
+    replaceAllUsesWith(module.get(), reluCall.getResult(0), call.getResult(0));
+    erased.insert(reluCall.op);
+    reluCall->erase();
+    relu.setAttr("func.state", "fused");
+  }
+
+  for (auto matmul : matmuls) {
+    matmul.setAttr("kcg.BLOCK_SIZE_M", std::to_string(cfg("BLOCK_SIZE_M", 128)));
+    matmul.setAttr("kcg.BLOCK_SIZE_N", std::to_string(cfg("BLOCK_SIZE_N", 128)));
+    matmul.setAttr("kcg.BLOCK_SIZE_K", std::to_string(cfg("BLOCK_SIZE_K", 8)));
+    matmul.setAttr("kcg.GROUP_SIZE_M", std::to_string(cfg("GROUP_SIZE_M", 8)));
+    matmul.setAttr("kcg.WAVE_SIZE_M", std::to_string(cfg("WAVE_SIZE_M", 64)));
+    matmul.setAttr("kcg.WAVE_SIZE_N", std::to_string(cfg("WAVE_SIZE_N", 64)));
+    matmul.setAttr("kcg.VECTORIZE_WIDTH", std::to_string(cfg("VECTORIZE_WIDTH", 4)));
+    matmul.setAttr("kcg.WARP_SIZE", std::to_string(cfg("WARP_SIZE", 64)));
+  }
+}
+
+// ------------------------------------------------------------------- FMHA
+bool FMHAOptimizer::applicable(ModuleOp &module) {
+  clear();
+  auto isCpuFunc = [&](const std::string &callee, const char *prefix) {
+    if (callee.find(prefix) == std::string::npos) return false;
+    FuncOp f = Analyzer::getTargetFunction(module, callee);
+    return f && f.getAttr("func.state") == "cpu";
+  };
+  auto onlyUserCall = [&](CallOp call) -> CallOp {
+    auto users = Analyzer::getUsers(module, call.getResult(0));
+    if (Analyzer::getUsersNumber(users) != 1 || users[0]->kind != OpKind::Call) return CallOp();
+    return CallOp(users[0]);
+  };
+  for (auto call2Matmul : Analyzer::collectFuncCalls(module)) {
+    if (!isCpuFunc(call2Matmul.getCallee(), "BatchMatmul")) continue;
+    CallOp call2Softmax = onlyUserCall(call2Matmul);
+    if (!call2Softmax || !isCpuFunc(call2Softmax.getCallee(), "Softmax")) continue;
+    CallOp call2Matmul2 = onlyUserCall(call2Softmax);
+    if (!call2Matmul2 || !isCpuFunc(call2Matmul2.getCallee(), "BatchMatmul")) continue;
+    if (uniqueFuncCalls.count(call2Matmul) || uniqueFuncCalls.count(call2Softmax) ||
+        uniqueFuncCalls.count(call2Matmul2))
+      continue;
+    MemoryBuffer buf;
+    if (!identifyBatchMatmul(call2Matmul.getCallee(), buf.matmul1) ||
+        !identifyBatchMatmul(call2Matmul2.getCallee(), buf.matmul2))
+      continue;
+    // S = Q.K^T ('N','T'), O = P.V ('N','N'), same batch, rows match, S columns = V rows,
+    // and P (the softmax result) is the left operand of the second product
+    if (buf.matmul1.transA || !buf.matmul1.transB || buf.matmul2.transA || buf.matmul2.transB) continue;
+    if (buf.matmul1.batch != buf.matmul2.batch || buf.matmul1.m != buf.matmul2.m ||
+        buf.matmul1.n != buf.matmul2.k)
+      continue;
+    if (call2Matmul2.getArgOperands()[0] != call2Softmax.getResult(0)) continue;
+    buf.Q = call2Matmul.getArgOperands()[0];
+    buf.K = call2Matmul.getArgOperands()[1];
+    buf.S = call2Matmul.getArgOperands()[2];
+    buf.V = call2Matmul2.getArgOperands()[1];
+    buf.O = call2Matmul2.getArgOperands()[2];
+    call2bufferMap[call2Matmul] = buf;
+    call2callsMap[call2Matmul] = {call2Softmax, call2Matmul2};
+    uniqueFuncCalls.insert(call2Matmul);
+    uniqueFuncCalls.insert(call2Softmax);
+    uniqueFuncCalls.insert(call2Matmul2);
+  }
+  return !call2callsMap.empty();
+}
+
+void FMHAOptimizer::applyOptimzer(ModuleOp &module) {
+  auto cfg = [&](const char *key, int fallback) {
+    auto it = fmhaConfig.find(key);
+    return it == fmhaConfig.end() ? fallback : it->second;
+  };
+  for (auto &item : call2callsMap) {
+    CallOp call2Matmul = item.first;
+    CallOp call2Softmax = item.second[0];
+    CallOp call2Matmul2 = item.second[1];
+    const MemoryBuffer &buf = call2bufferMap[call2Matmul];
+    const BatchMatmulDescriptor &d1 = buf.matmul1;
+    const int seq_len = d1.m, head_dim = d1.k;
+
+    std::string fusedFuncName = "Fused_Multi_Head_Attention";
+    for (auto b : d1.batch) fusedFuncName += "_" + std::to_string(b);
+    fusedFuncName += "_SL" + std::to_string(seq_len) + "_HD" + std::to_string(head_dim);
+
+    const int Hd = head_dim;
+    int Br = cfg("Br", 0), Bc = cfg("Bc", 0);
+    if (Br == 0) Br = cfg("HdxBr", 128 * 128) / Hd;   // the reference's derivation
+    if (Bc == 0) Bc = cfg("BrxBc", 128 * 32) / Br;
+    const int blockSize = cfg("BLOCK_SIZE", 256);
+    fmhaConfig["Hd"] = Hd;
+    fmhaConfig["Br"] = Br;
+    fmhaConfig["Bc"] = Bc;
+
+    const MemRefType tq = buf.Q.getMemRefType(), tk = buf.K.getMemRefType(), tv = buf.V.getMemRefType(),
+                     to = buf.O.getMemRefType();
+    FuncOp funcOp = buildFuction(module, fusedFuncName, {tq, tk, tv, to}, {to});
+    Op *newCall = call2Matmul2->insertAfter(makeCall(funcOp.op, {buf.Q, buf.K, buf.V, buf.O}));
+    replaceAllUsesWith(module.get(), call2Matmul2.getResult(0), newCall->result(0));
+    call2Matmul2->erase();
+    call2Softmax->erase();
+    call2Matmul->erase();
+    // the S buffer has no reader left
+    if (Op *sDef = buf.S.getDefiningOp())
+      if (Analyzer::getUsers(module, buf.S).empty()) sDef->erase();
+
+    if (funcOp->body.empty()) {
+      auto args = funcOp.getArguments();
+      funcOp->pushBack(makeReturn({args[3]}));
+      // grid (batch.., ceil(S / Br)) x block (BLOCK_SIZE): one loop per level dimension,
+      // then the same for -> parallel conversion the matmul recipe uses.
+      // affine.parallel carries at most three dimensions (X, Y, Z): with more than
+      // two batch dimensions they are folded into one
+      std::vector<int64_t> bounds;
+      if (d1.batch.size() <= 2) {
+        for (auto b : d1.batch) bounds.push_back(b);
+      } else {
+        int64_t all = 1;
+        for (auto b : d1.batch) all *= b;
+        bounds.push_back(all);
+      }
+      bounds.push_back((seq_len + Br - 1) / Br);
+      std::vector<ForOp> gridLoops;
+      Op *cur = funcOp.op;
+      for (auto b : bounds) {
+        ForOp l = Rewriter::create_constant_loop(OpHandle(cur), 0, b, 1);
+        gridLoops.push_back(l);
+        cur = l.op;
+      }
+      ForOp blockLoop = Rewriter::create_constant_loop(OpHandle(cur), 0, blockSize, 1);
+      auto gridLevel = Rewriter::parallel(gridLoops);
+      auto blockLevel = Rewriter::parallel({blockLoop});
+      const DType elem = tq.elem;
+      // LDS tiles of the gfx950 kernel: K as [Bc][Hd + pad], V as [Bc][Hd + pad]
+      const int padK = elem == DType::f32 ? 4 : 8, padV = elem == DType::f32 ? 8 : 32;
+      Rewriter::alloc_buffer(OpHandle(gridLevel.op), MemorySpace::shared, {Bc, Hd + padV}, elem);
+      Rewriter::alloc_buffer(OpHandle(gridLevel.op), MemorySpace::shared, {Bc, Hd + padK}, elem);
+      // per-lane registers: O^T accumulators (Hd/32 MFMA blocks x 16) and the running max / sum
+      Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {2}, DType::f32);
+      Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {Hd / 32 > 0 ? Hd / 32 : 1, 16}, DType::f32);
+      funcOp.setAttr("func.state", "gpu");
+      funcOp.setAttr("kcg.Br", std::to_string(Br));
+      funcOp.setAttr("kcg.Bc", std::to_string(Bc));
+      funcOp.setAttr("kcg.Hd", std::to_string(Hd));
+      funcOp.setAttr("kcg.BLOCK_SIZE", std::to_string(blockSize));
+      char sc[64];
+      snprintf(sc, sizeof sc, "%.9g", static_cast<double>(scale));
+      funcOp.setAttr("kcg.scale", sc);
+      funcOp.setAttr("kcg.causal", causal ? "1" : "0");
+    }
+    DUMP(module);
+  }
+  // the three un-fused functions may have no caller left
+  for (auto f : Analyzer::collectFunctions(module)) {
+    if (f.getAttr("func.state") != "cpu") continue;
+    bool called = false;
+    for (auto c : Analyzer::collectFuncCalls(module)) called = called || c.getCallee() == f.getSymName();
+    if (!called) f->erase();
+  }
+}
+
+}  // namespace KernelCodeGen

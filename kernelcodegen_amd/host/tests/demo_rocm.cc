@@ -1,0 +1,126 @@
+// GPU demo of the host layer: the reference's test_matmul / test_flash_attention
+// flows (test/test.cc:8-107 there) carried through to a launch on the device.
+//
+//   demo_rocm matmul M N K relu(0|1) out.bin
+//   demo_rocm fmha   B H S D causal(0|1) scale out.bin
+//
+// Builds the graph through KernelCodeGenerator, optimizes it, binds the result
+// to the gfx950 kernel, runs it on seeded uniform[-1,1) inputs (the generator of
+// kernelcodegen_amd/inputs.py: splitmix64 of seed ^ tensor<<56 ^ index, top 24
+// bits), and writes the raw fp32 output to out.bin for the caller to check.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "KernelCodeGen.h"
+
+using namespace KernelCodeGen;
+
+static const uint64_t kSeed = 0xD3A0;
+
+static void fill_uniform(std::vector<float> &v, uint64_t seed, uint64_t tensor) {
+  for (size_t i = 0; i < v.size(); ++i) {
+    uint64_t x = (seed ^ (tensor << 56) ^ static_cast<uint64_t>(i)) + 0x9E3779B97F4A7C15ull;
+    uint64_t z = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    v[i] = static_cast<float>(static_cast<double>(z >> 40) / 8388608.0 - 1.0);
+  }
+}
+
+#define HIP_OK(call)                                                             \
+  do {                                                                           \
+    hipError_t e_ = (call);                                                      \
+    if (e_ != hipSuccess) {                                                      \
+      std::fprintf(stderr, "%s failed: %s\n", #call, hipGetErrorString(e_));     \
+      return 2;                                                                  \
+    }                                                                            \
+  } while (0)
+
+static int run(const KernelBinding &b, const std::vector<std::vector<float> *> &inputs, size_t outCount,
+               const char *outPath) {
+  std::vector<void *> dev;
+  for (auto *h : inputs) {
+    void *d = nullptr;
+    HIP_OK(hipMalloc(&d, h->size() * sizeof(float)));
+    HIP_OK(hipMemcpy(d, h->data(), h->size() * sizeof(float), hipMemcpyHostToDevice));
+    dev.push_back(d);
+  }
+  void *out = nullptr;
+  HIP_OK(hipMalloc(&out, outCount * sizeof(float)));
+  HIP_OK(hipMemset(out, 0xFF, outCount * sizeof(float)));
+  dev.push_back(out);
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  const int st = HIPLaunch(b, dev, stream);
+  if (st != KCG_OK) {
+    std::fprintf(stderr, "launch failed: %s\n", kcg_status_str(st));
+    return 3;
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+  std::vector<float> host(outCount);
+  HIP_OK(hipMemcpy(host.data(), out, outCount * sizeof(float), hipMemcpyDeviceToHost));
+  FILE *fp = std::fopen(outPath, "wb");
+  if (!fp) return 4;
+  std::fwrite(host.data(), sizeof(float), host.size(), fp);
+  std::fclose(fp);
+  for (void *d : dev) HIP_OK(hipFree(d));
+  HIP_OK(hipStreamDestroy(stream));
+  return 0;
+}
+
+int main(int argc, char **argv) {
+  if (argc < 2) {
+    std::fprintf(stderr, "usage: demo_rocm matmul M N K relu out | demo_rocm fmha B H S D causal scale out\n");
+    return 1;
+  }
+  KernelCodeGenerator generator("ROCm");
+  generator.setLogMode(Log::Release);
+  const std::string mode = argv[1];
+  if (mode == "matmul" && argc == 7) {
+    const int64_t m = std::atoll(argv[2]), n = std::atoll(argv[3]), k = std::atoll(argv[4]);
+    const bool relu = std::atoi(argv[5]) != 0;
+    auto &graph = generator.createGraph("matmul_demo");
+    auto A = graph.create<PlaceHolder>(std::vector<int64_t>{m, k}, std::string{"float32"});
+    auto B = graph.create<PlaceHolder>(std::vector<int64_t>{k, n}, std::string{"float32"});
+    auto C = graph.create<Matmul>(A, B, MemorySpace::global);
+    if (relu) graph.create<Relu>(C, MemorySpace::inplace);
+    auto module = generator.optimize(graph);
+    auto bindings = generator.bind(module);
+    if (bindings.size() != 1) return 5;
+    std::printf("%s", generator.codegen(module).c_str());
+    std::vector<float> a(m * k), b(k * n);
+    fill_uniform(a, kSeed, 0);
+    fill_uniform(b, kSeed, 1);
+    return run(bindings[0], {&a, &b}, static_cast<size_t>(m * n), argv[6]);
+  }
+  if (mode == "fmha" && argc == 9) {
+    const int64_t bsz = std::atoll(argv[2]), h = std::atoll(argv[3]), s = std::atoll(argv[4]), d = std::atoll(argv[5]);
+    FMHAOptimizer::causal = std::atoi(argv[6]) != 0;
+    FMHAOptimizer::scale = static_cast<float>(std::atof(argv[7]));
+    auto &graph = generator.createGraph("flash_attn_demo");
+    std::vector<int64_t> shape{bsz, h, s, d};
+    auto Q = graph.create<PlaceHolder>(shape, std::string{"float32"});
+    auto K = graph.create<PlaceHolder>(shape, std::string{"float32"});
+    auto V = graph.create<PlaceHolder>(shape, std::string{"float32"});
+    auto S = graph.create<BatchedMatmul>(Q, Layout::rowMajor, K, Layout::colMajor);
+    auto P = graph.create<Softmax>(S, -1, MemorySpace::inplace);
+    graph.create<BatchedMatmul>(P, Layout::rowMajor, V, Layout::rowMajor);
+    auto module = generator.optimize(graph);
+    auto bindings = generator.bind(module);
+    if (bindings.size() != 1) return 5;
+    std::printf("%s", generator.codegen(module).c_str());
+    const size_t count = static_cast<size_t>(bsz * h * s * d);
+    std::vector<float> q(count), kk(count), v(count);
+    fill_uniform(q, kSeed, 0);
+    fill_uniform(kk, kSeed, 1);
+    fill_uniform(v, kSeed, 2);
+    return run(bindings[0], {&q, &kk, &v}, count, argv[8]);
+  }
+  std::fprintf(stderr, "bad arguments\n");
+  return 1;
+}

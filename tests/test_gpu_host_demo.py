@@ -1,0 +1,49 @@
+"""The C++ host layer end to end on the GPU: graph -> optimize -> bind -> launch
+(kernelcodegen_amd/host/tests/demo_rocm.cc, the reference's test_matmul /
+test_flash_attention flows), checked against the oracle."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import rel_err
+from kernelcodegen_amd import inputs
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEMO = os.path.join(ROOT, "kernelcodegen_amd", "host", "demo_rocm")
+SEED = 0xD3A0
+
+
+def _run(args, tmp_path):
+    if not os.path.exists(DEMO):
+        pytest.fail("kernelcodegen_amd/host/demo_rocm is not built (run __graft_entry__.build())")
+    out = str(tmp_path / "out.bin")
+    res = subprocess.run([DEMO] + [str(a) for a in args] + [out], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
+    return np.fromfile(out, dtype=np.float32), res.stdout
+
+
+@pytest.mark.parametrize("shape,relu", [((512, 384, 256), 1), ((4096, 2048, 1024), 1), ((200, 136, 52), 0)])
+def test_matmul_demo(oracle, dev, tmp_path, shape, relu):
+    M, N, K = shape
+    got, text = _run(["matmul", M, N, K, relu], tmp_path)
+    assert "namespace matmul_demo {" in text and "kcg_gemm_f32(arg0, arg1, arg2, %d, %d, %d" % (M, N, K) in text
+    A = inputs.uniform((M, K), SEED, 0)
+    B = inputs.uniform((K, N), SEED, 1)
+    ref = oracle.matmul(A, B)
+    if relu:
+        ref = oracle.relu(ref)
+    assert max(rel_err(got.reshape(M, N), ref)) < 1e-4
+
+
+@pytest.mark.parametrize("causal", [0, 1])
+def test_flash_attention_demo(oracle, dev, tmp_path, causal):
+    B, H, S, D = 2, 4, 384, 64
+    scale = 0.125
+    got, text = _run(["fmha", B, H, S, D, causal, scale], tmp_path)
+    assert "kcg_fmha_f32(arg0, arg1, arg2, arg3, 2, 4, 384, 64, 0.125f, %d" % causal in text
+    Q, K, V = (inputs.uniform((B, H, S, D), SEED, i) for i in range(3))
+    ref = oracle.fmha(Q, K, V, scale=scale, causal=bool(causal), stable=True)
+    assert max(rel_err(got.reshape(B, H, S, D), ref)) < 1e-4
