@@ -8,7 +8,7 @@
 // and causal mask.
 //
 // Work split: 4 waves per workgroup, QT*32 query rows per wave (Br = 128*QT),
-// K/V swept in tiles of BC rows.
+// K/V swept in tiles of BC = 64 rows.
 //
 //  * S^T = K . Q^T: A operand = K rows from LDS (one ds_read_b128 = 8 bf16 of d
 //    per lane), B operand = Q, held in registers for the whole sweep.  Lane
@@ -21,13 +21,29 @@
 //    its natural [key][d] LDS layout with two ds_read_b64_tr_b16 per MFMA: in
 //    each group of 16 lanes, source lane L addresses V[k0 + L/4][d0 + 4*(L%4)..+3]
 //    and destination lane i receives keys k0..k0+3 of column d0 + i.
-//
-// LDS (bf16 elements): Ks[BC][D+8]   pitch = 4 banks mod 64: b128 reads of 16
-//                                    consecutive rows are conflict free
-//                      Vs[BC][D+32]  pitch = 16 banks mod 64: the 4 rows x 32 B
-//                                    touched by one 16-lane transpose group, and
-//                                    the neighbouring group 32 B further, are
-//                                    bank-disjoint
+//  * K/V tiles go from global memory straight into LDS (global_load_lds_dwordx4,
+//    no staging registers, no LDS store instructions): one wave instruction fills
+//    1024 consecutive LDS bytes, lane L supplying the 16-byte chunk that belongs
+//    at position L.  Rows are therefore unpadded; bank conflicts are avoided by
+//    an XOR swizzle of the 16-byte chunk index, applied to the *global* address
+//    when loading and to the LDS address when reading:
+//        K: chunk c of row r sits at c ^ fk(r)   (16 consecutive rows, same c,
+//                                                  hit 16 distinct 16-byte slots)
+//        V: chunk c of row r sits at c ^ fv(r)   (the 4 rows x 32 B of one
+//                                                  16-lane transpose group, and
+//                                                  the neighbouring group, are
+//                                                  slot-disjoint)
+//    The buffers are double-buffered: tile t+1 streams in while tile t is
+//    consumed; each wave waits for its own loads (vmcnt) before the single
+//    barrier that ends the step.
+//  * Online softmax in base 2 with a lazy rescale: the running reference maximum
+//    of a row is only raised (and O, l rescaled) when the tile maximum exceeds it
+//    by more than kTau; exp2(s*c - m) is one FMA + v_exp_f32; row sums use
+//    v_dot2c_f32_bf16 on the packed P.
+//  * Causal: a workgroup runs the query-block pair (n-1-i, i), so all workgroups
+//    sweep the same number of tiles; tiles above a wave's last row are skipped.
+#include <type_traits>
+
 #include "kcg_common.h"
 
 namespace kcg {
@@ -39,21 +55,28 @@ typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 
 #define KCG_LDS_BF16X4 __attribute__((address_space(3))) bf16x4_v
+#define KCG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define KCG_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 template <int D, int BC, int QT>
 struct FmhaBf16Tile {
   static constexpr int kThreads = 256;
   static constexpr int kBr = 128 * QT;
   static constexpr int kWaveRows = 32 * QT;
-  static constexpr int kPitchK = D + 8;
-  static constexpr int kPitchV = D + 32;
-  static constexpr int kLdsBytes = (BC * kPitchK + BC * kPitchV) * 2;
-  static constexpr int kLoads = BC * D / 8 / kThreads;  // 16-byte loads per thread per tile
+  static constexpr int kCpr = D / 8;            // 16-byte chunks per row
+  static constexpr int kRowsPer256 = 16 / kCpr;  // rows that share one 256-byte bank window
+  static constexpr int kRpi = 64 / kCpr;         // rows filled by one wave-wide direct load
+  static constexpr int kIpw = BC / kRpi / 4;     // direct loads per wave per tile
+  static constexpr int kTile = BC * D;           // elements per K (or V) buffer, unpadded
+  static constexpr int kLdsBytes = 2 * 2 * kTile * 2;  // K and V, double-buffered
   static constexpr int kKeyTiles = BC / 32;
   static constexpr int kDTiles = D / 32;
   static constexpr int kDSteps = D / 16;
-  static_assert(BC % 32 == 0 && D % 32 == 0, "tile extents");
-  static_assert((BC * D / 8) % kThreads == 0, "load split");
+  static_assert(D == 64 || D == 128, "head dim");
+  static_assert(BC % (4 * kRpi) == 0 && BC % 32 == 0, "tile extents");
+  // chunk-index swizzles (see the file header)
+  __host__ __device__ static constexpr int fk(int row) { return (row / kRowsPer256) % kCpr; }
+  __host__ __device__ static constexpr int fv(int row) { return 4 * ((row / kRowsPer256) & (kCpr / 4 - 1)); }
 };
 
 __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
@@ -63,23 +86,38 @@ __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
   return __builtin_bit_cast(unsigned, r);
 }
 
-template <int D, int BC, int QT, bool CAUSAL, bool OUT_BF16>
+// a.x + a.y + acc for a packed bf16 pair (v_dot2c_f32_bf16 with a pair of ones).
+__device__ __forceinline__ float add_bf16_pair(unsigned pair, float acc) {
+  const bf16x2_v ones = {static_cast<__bf16>(1.0f), static_cast<__bf16>(1.0f)};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, pair), ones, acc, false);
+}
+
+// How far (in log2 units) a tile's row maximum may exceed the running reference
+// before the accumulators are rescaled.  Between rescales P is at most 2^kTau,
+// harmless for bf16 P (relative precision is scale free) and fp32 sums; the final
+// O / l normalisation is exact for any reference.
+constexpr float kTau = 8.0f;
+
+// POS_SCALE: scale > 0, so exp2(s * c - m) is one FMA and the row maximum can be
+// taken on the raw products.  The general variant scales first.
+template <int D, int BC, int QT, bool CAUSAL, bool OUT_BF16, bool POS_SCALE>
 __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
-    void *__restrict__ O, int S, int q_blocks, float scale_log2e) {
+    void *__restrict__ O, int S, int q_blocks, int q_items, float scale_log2e) {
   using T = FmhaBf16Tile<D, BC, QT>;
   extern __shared__ __align__(16) uint16_t lds16[];
-  uint16_t *Ks = lds16;
-  uint16_t *Vs = lds16 + BC * T::kPitchK;
+  uint16_t *Ks = lds16;                  // [2][BC][D], chunk-swizzled
+  uint16_t *Vs = lds16 + 2 * T::kTile;   // [2][BC][D], chunk-swizzled
 
-  // Every XCD walks a contiguous range of (head, query block) ids, head-major, so
-  // the K/V of a head are fetched into one XCD's L2 only; heavy (late) query
-  // blocks first when causal.
+  // Every XCD walks a contiguous range of (head, work item) ids, head-major, so
+  // the K/V of a head are fetched into one XCD's L2 only.  Causal: a work item is
+  // the pair of query blocks (n-1-i, i), so every workgroup sweeps the same
+  // number of K/V tiles and the grid has no heavy tail.
   const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int qb_raw = bid % q_blocks;
-  const int bh = bid / q_blocks;
-  const int qb = CAUSAL ? (q_blocks - 1 - qb_raw) : qb_raw;
-  const int q0 = qb * T::kBr;
+  const int bh = bid / q_items;
+  const int item = bid - bh * q_items;
+  const int hi_block = q_blocks - 1 - item;
+  const int npass = CAUSAL ? (hi_block != item ? 2 : 1) : 1;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -92,213 +130,306 @@ __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
   const uint16_t *Kb = K + base;
   const uint16_t *Vb = V + base;
 
-  const int wq0 = q0 + wave * T::kWaveRows;  // first query row of this wave
-
-  // ---- Q fragments: q[qt][s] = Q[wq0 + 32*qt + r32][16*s + 8*half .. +7] ----
-  bf16x8_v q[QT][T::kDSteps];
+  // ---- direct global -> LDS tile loads ----
+  // Wave instruction j of this wave fills LDS rows ld_row0 + j*kRpi .. +kRpi-1; lane L
+  // sits at row ld_row0 + j*kRpi + L / kCpr, chunk position L % kCpr, and fetches the
+  // global chunk (position ^ swizzle(row)) of that row.
+  const int ld_row0 = wave * T::kIpw * T::kRpi;
+  const int ld_lrow = lane / T::kCpr;
+  const int ld_pos = lane % T::kCpr;
+  int goff_k[T::kIpw], goff_v[T::kIpw];  // element offsets inside a tile, per instruction
 #pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    const int row = wq0 + 32 * qt + r32;
-#pragma unroll
-    for (int s = 0; s < T::kDSteps; ++s) {
-      u32x4_t v = {0u, 0u, 0u, 0u};
-      if (row < S)
-        v = *reinterpret_cast<const u32x4_t *>(Qb + static_cast<int64_t>(row) * D + 16 * s + 8 * half);
-      q[qt][s] = __builtin_bit_cast(bf16x8_v, v);
-    }
+  for (int j = 0; j < T::kIpw; ++j) {
+    const int row = ld_row0 + j * T::kRpi + ld_lrow;
+    goff_k[j] = row * D + (ld_pos ^ T::fk(row)) * 8;
+    goff_v[j] = row * D + (ld_pos ^ T::fv(row)) * 8;
   }
-
-  float16_t acc_o[QT][T::kDTiles];
+  auto load_tiles = [&](int kv0, int buf) {
+    const uint16_t *kg = Kb + static_cast<int64_t>(kv0) * D;
+    const uint16_t *vg = Vb + static_cast<int64_t>(kv0) * D;
+    uint16_t *kl = Ks + buf * T::kTile + ld_row0 * D;
+    uint16_t *vl = Vs + buf * T::kTile + ld_row0 * D;
+    if (kv0 + BC <= S) {
 #pragma unroll
-  for (int qt = 0; qt < QT; ++qt)
+      for (int j = 0; j < T::kIpw; ++j) {
+        __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(kg + goff_k[j]), KCG_LDS_PTR(kl + j * T::kRpi * D), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(vg + goff_v[j]), KCG_LDS_PTR(vl + j * T::kRpi * D), 16, 0, 0);
+      }
+    } else {
+      // ragged last tile: rows at and beyond S are zero-filled, through registers
 #pragma unroll
-    for (int i = 0; i < T::kDTiles; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc_o[qt][i][e] = 0.0f;
-  float m_run[QT], l_run[QT];
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    m_run[qt] = -INFINITY;
-    l_run[qt] = 0.0f;
-  }
-
-  const int kv_end = CAUSAL ? ((q0 + T::kBr) < S ? (q0 + T::kBr) : S) : S;
-  const int n_tiles = (kv_end + BC - 1) / BC;
-
-  u32x4_t stage[T::kLoads];
-  auto load_tile = [&](const uint16_t *src, int kv0) {
-#pragma unroll
-    for (int i = 0; i < T::kLoads; ++i) {
-      const int idx = tid + i * T::kThreads;
-      const int row = idx / (D / 8);
-      const int c8 = idx % (D / 8);
-      u32x4_t v = {0u, 0u, 0u, 0u};
-      if (kv0 + row < S)
-        v = *reinterpret_cast<const u32x4_t *>(src + static_cast<int64_t>(kv0 + row) * D + c8 * 8);
-      stage[i] = v;
+      for (int j = 0; j < T::kIpw; ++j) {
+        const int row = ld_row0 + j * T::kRpi + ld_lrow;
+        const bool ok = kv0 + row < S;
+        const u32x4_t z = {0u, 0u, 0u, 0u};
+        const u32x4_t kvq = ok ? *reinterpret_cast<const u32x4_t *>(kg + goff_k[j]) : z;
+        const u32x4_t vvq = ok ? *reinterpret_cast<const u32x4_t *>(vg + goff_v[j]) : z;
+        *reinterpret_cast<u32x4_t *>(kl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = kvq;
+        *reinterpret_cast<u32x4_t *>(vl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = vvq;
+      }
     }
   };
-  auto store_tile = [&](uint16_t *dst, int pitch) {
-#pragma unroll
-    for (int i = 0; i < T::kLoads; ++i) {
-      const int idx = tid + i * T::kThreads;
-      const int row = idx / (D / 8);
-      const int c8 = idx % (D / 8);
-      *reinterpret_cast<u32x4_t *>(dst + row * pitch + c8 * 8) = stage[i];
-    }
+  // Every wave waits for its own direct loads; the barrier then publishes all of them.
+  auto tiles_ready = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
   };
 
-  // Per-lane constant part of the V transpose-read address (elements):
-  // row offset 4*half + (lane%16)/4, column 16*((lane/16)%2) + 4*(lane%4).
+  // ---- per-lane read addresses (elements), swizzle folded in ----
+  // K fragment of d-step ds: row r32 (+32*kt), chunk (2*ds + half) ^ fk(row)
+  const int k_row_off = r32 * D;
+  const int k_swz = T::fk(r32) ^ half;  // chunk position = (2*ds) ^ k_swz
+  // V transpose read: row 4*half + (lane%16)/4 (+8u + 16b + 32kt), column
+  // 32*i + 16*((lane/16)%2) + 4*(lane%4): chunk 4*i + (v_c0 ^ ...), 8-byte half v_sub
   const int l16 = lane & 15;
-  const int vtr_off = (4 * half + (l16 >> 2)) * T::kPitchV + 16 * ((lane >> 4) & 1) + 4 * (l16 & 3);
+  const int v_lrow = 4 * half + (l16 >> 2);
+  const int v_c0 = (2 * ((lane >> 4) & 1) + ((l16 & 3) >> 1)) ^ T::fv(v_lrow);  // chunk = (4*i) ^ v_c0
+  const int v_sub = 4 * (l16 & 1);
+  const int v_row_off = v_lrow * D + v_sub;
 
-  load_tile(Kb, 0);
-  store_tile(Ks, T::kPitchK);
-  __syncthreads();
+#pragma unroll 1
+  for (int pass = 0; pass < npass; ++pass) {
+    const int qb = CAUSAL ? (pass == 0 ? hi_block : item) : item;
+    const int q0 = qb * T::kBr;
+    const int wq0 = q0 + wave * T::kWaveRows;  // first query row of this wave
 
-  for (int t = 0; t < n_tiles; ++t) {
-    const int kv0 = t * BC;
-    load_tile(Vb, kv0);
+    // ---- Q fragments: q[qt][s] = Q[wq0 + 32*qt + r32][16*s + 8*half .. +7] ----
+    bf16x8_v q[QT][T::kDSteps];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      const int row = wq0 + 32 * qt + r32;
+#pragma unroll
+      for (int s = 0; s < T::kDSteps; ++s) {
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        if (row < S)
+          v = *reinterpret_cast<const u32x4_t *>(Qb + static_cast<int64_t>(row) * D + 16 * s + 8 * half);
+        q[qt][s] = __builtin_bit_cast(bf16x8_v, v);
+      }
+    }
 
-    // ---- S^T = K . Q^T ----
-    float16_t s[QT][T::kKeyTiles];
+    float16_t acc_o[QT][T::kDTiles];
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
-      for (int kt = 0; kt < T::kKeyTiles; ++kt)
+      for (int i = 0; i < T::kDTiles; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s[qt][kt][e] = 0.0f;
+        for (int e = 0; e < 16; ++e) acc_o[qt][i][e] = 0.0f;
+    float m_ref[QT], l_run[QT];  // reference maximum (log2 units), this lane's share of the row sum
 #pragma unroll
-    for (int kt = 0; kt < T::kKeyTiles; ++kt) {
-      const uint16_t *kp = Ks + (kt * 32 + r32) * T::kPitchK + 8 * half;
-#pragma unroll
-      for (int ds = 0; ds < T::kDSteps; ++ds) {
-        const bf16x8_v kf =
-            __builtin_bit_cast(bf16x8_v, *reinterpret_cast<const u32x4_t *>(kp + 16 * ds));
-#pragma unroll
-        for (int qt = 0; qt < QT; ++qt)
-          s[qt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q[qt][ds], s[qt][kt], 0, 0, 0);
-      }
+    for (int qt = 0; qt < QT; ++qt) {
+      m_ref[qt] = -INFINITY;
+      l_run[qt] = 0.0f;
     }
 
-    // ---- scale, mask, online softmax (base 2) ----
-    unsigned p[QT][T::kKeyTiles][8];  // bf16 pairs: word w packs P elements 2w, 2w+1
+    const int kv_end = CAUSAL ? ((q0 + T::kBr) < S ? (q0 + T::kBr) : S) : S;
+    const int n_tiles = (kv_end + BC - 1) / BC;
+
+    load_tiles(0, 0);
+    tiles_ready();
+
+    for (int t = 0; t < n_tiles; ++t) {
+      const int kv0 = t * BC;
+      const int cur = t & 1;
+      if (t + 1 < n_tiles) load_tiles(kv0 + BC, cur ^ 1);  // streams in while this tile is computed
+
+      // A wave whose last query precedes the tile has nothing to add (causal).
+      const bool wave_active = !CAUSAL || (kv0 <= wq0 + T::kWaveRows - 1);
+      if (wave_active) {
+        const uint16_t *ks = Ks + cur * T::kTile + k_row_off;
+        const uint16_t *vs = Vs + cur * T::kTile + v_row_off;
+
+        // ---- S^T = K . Q^T ----
+        float16_t s[QT][T::kKeyTiles];
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+          for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[qt][kt][e] = 0.0f;
+        {
+          // K fragments are requested two d-steps ahead of the MFMAs that use them
+          constexpr int kAhead = 2;
+          bf16x8_v kf[T::kDSteps][T::kKeyTiles];
+          auto fetch = [&](int ds) {
+#pragma unroll
+            for (int kt = 0; kt < T::kKeyTiles; ++kt)
+              kf[ds][kt] = __builtin_bit_cast(
+                  bf16x8_v, *reinterpret_cast<const u32x4_t *>(ks + kt * 32 * D + ((2 * ds) ^ k_swz) * 8));
+          };
+#pragma unroll
+          for (int ds = 0; ds < kAhead; ++ds) fetch(ds);
+#pragma unroll
+          for (int ds = 0; ds < T::kDSteps; ++ds) {
+            if (ds + kAhead < T::kDSteps) fetch(ds + kAhead);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+              for (int qt = 0; qt < QT; ++qt)
+                s[qt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds][kt], q[qt][ds], s[qt][kt], 0, 0, 0);
+          }
+        }
+
+        // ---- mask, online softmax (base 2, lazy rescale) ----
+        unsigned p[QT][T::kKeyTiles][8];  // bf16 pairs: word w packs P elements 2w, 2w+1
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+          const int qrow = wq0 + 32 * qt + r32;
+          const bool need_mask = (kv0 + BC > S) || (CAUSAL && (kv0 + BC - 1 > wq0 + 32 * qt));
+          if (POS_SCALE) {
+            // fast path: exp2(s * c - m) as one FMA; the maximum is taken on raw S
+            if (need_mask) {
+              // element (kt, e) is key kv0 + 4*half + off, off = 32*kt + 8*(e/4) + e%4;
+              // it is dead when off > lim
+              const int last = CAUSAL ? (qrow < S - 1 ? qrow : S - 1) : (S - 1);
+              const int lim = last - kv0 - 4 * half;
+#pragma unroll
+              for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                  if (32 * kt + 8 * (e / 4) + (e % 4) > lim) s[qt][kt][e] = -INFINITY;
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[qt][kt][e]);
+            float m_loc = mx * scale_log2e;  // -inf stays -inf
+            m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
+            // per-row decision: a row's result never depends on what other rows do
+            if (m_loc > m_ref[qt] + kTau) {
+              const float m_new = fmaxf(m_ref[qt], m_loc);
+              const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+              const float alpha = __builtin_amdgcn_exp2f(m_ref[qt] - m_use);  // m_ref = -inf -> 0
+              l_run[qt] *= alpha;
+              m_ref[qt] = m_new;
+#pragma unroll
+              for (int i = 0; i < T::kDTiles; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc_o[qt][i][e] *= alpha;
+            }
+            const float neg_m = (m_ref[qt] == -INFINITY) ? 0.0f : -m_ref[qt];
+            float psum = 0.0f;
+#pragma unroll
+            for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+              for (int w = 0; w < 8; ++w) {
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qt][kt][2 * w], scale_log2e, neg_m));
+                const float p1 =
+                    __builtin_amdgcn_exp2f(__builtin_fmaf(s[qt][kt][2 * w + 1], scale_log2e, neg_m));
+                const unsigned pk = pack_bf16(p0, p1);
+                p[qt][kt][w] = pk;
+                psum = add_bf16_pair(pk, psum);
+              }
+            l_run[qt] += psum;
+          } else {
+            // general path (scale <= 0): scale first, then mask and maximum
+#pragma unroll
+            for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) s[qt][kt][e] *= scale_log2e;
+            if (need_mask) {
+#pragma unroll
+              for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                  const int key = kv0 + kt * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+                  if ((key >= S) || (CAUSAL && key > qrow)) s[qt][kt][e] = -INFINITY;
+                }
+            }
+            float m_loc = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) m_loc = fmaxf(m_loc, s[qt][kt][e]);
+            m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
+            const float m_new = fmaxf(m_ref[qt], m_loc);
+            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_ref[qt] - m_use);
+            float psum = 0.0f;
+#pragma unroll
+            for (int kt = 0; kt < T::kKeyTiles; ++kt)
+#pragma unroll
+              for (int w = 0; w < 8; ++w) {
+                const float p0 = __builtin_amdgcn_exp2f(s[qt][kt][2 * w] - m_use);
+                const float p1 = __builtin_amdgcn_exp2f(s[qt][kt][2 * w + 1] - m_use);
+                const unsigned pk = pack_bf16(p0, p1);
+                p[qt][kt][w] = pk;
+                psum = add_bf16_pair(pk, psum);
+              }
+            l_run[qt] = l_run[qt] * alpha + psum;
+            m_ref[qt] = m_new;
+#pragma unroll
+            for (int i = 0; i < T::kDTiles; ++i)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) acc_o[qt][i][e] *= alpha;
+          }
+        }
+
+        // ---- O^T += V^T . P^T ----
+#pragma unroll
+        for (int kt = 0; kt < T::kKeyTiles; ++kt) {
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const uint16_t *vp = vs + (kt * 32 + 16 * b) * D;
+#pragma unroll
+            for (int i = 0; i < T::kDTiles; ++i) {
+              const int col = ((4 * i) ^ v_c0) * 8;
+              const bf16x4_v lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((KCG_LDS_BF16X4 *)(vp + col));
+              const bf16x4_v hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((KCG_LDS_BF16X4 *)(vp + 8 * D + col));
+              const bf16x8_v vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+              for (int qt = 0; qt < QT; ++qt) {
+                const u32x4_t pw = {p[qt][kt][4 * b], p[qt][kt][4 * b + 1], p[qt][kt][4 * b + 2],
+                                    p[qt][kt][4 * b + 3]};
+                acc_o[qt][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    vf, __builtin_bit_cast(bf16x8_v, pw), acc_o[qt][i], 0, 0, 0);
+              }
+            }
+          }
+        }
+      }
+
+      tiles_ready();  // next tiles visible; every wave is done with the current buffers
+    }
+
+    // ---- normalise and store: lane holds O[qrow][32*i + 8*g + 4*half + 0..3] ----
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
       const int qrow = wq0 + 32 * qt + r32;
-      const bool need_mask = (kv0 + BC > S) || (CAUSAL && (kv0 + BC - 1 > wq0 + 32 * qt));
+      const float l_tot = l_run[qt] + __shfl_xor(l_run[qt], 32);
+      const float inv = 1.0f / l_tot;
+      if (qrow < S) {
+        const int64_t off = base + static_cast<int64_t>(qrow) * D + 4 * half;
 #pragma unroll
-      for (int kt = 0; kt < T::kKeyTiles; ++kt)
+        for (int i = 0; i < T::kDTiles; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s[qt][kt][e] *= scale_log2e;
-      if (need_mask) {
-#pragma unroll
-        for (int kt = 0; kt < T::kKeyTiles; ++kt)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int key = kv0 + kt * 32 + 8 * (e / 4) + 4 * half + (e % 4);
-            const bool dead = (key >= S) || (CAUSAL && key > qrow);
-            if (dead) s[qt][kt][e] = -INFINITY;
+          for (int g = 0; g < 4; ++g) {
+            const float v0 = acc_o[qt][i][4 * g + 0] * inv;
+            const float v1 = acc_o[qt][i][4 * g + 1] * inv;
+            const float v2 = acc_o[qt][i][4 * g + 2] * inv;
+            const float v3 = acc_o[qt][i][4 * g + 3] * inv;
+            if (OUT_BF16) {
+              u32x2_t w = {pack_bf16(v0, v1), pack_bf16(v2, v3)};
+              *reinterpret_cast<u32x2_t *>(static_cast<uint16_t *>(O) + off + 32 * i + 8 * g) = w;
+            } else {
+              float4_t w = {v0, v1, v2, v3};
+              *reinterpret_cast<float4_t *>(static_cast<float *>(O) + off + 32 * i + 8 * g) = w;
+            }
           }
       }
-      float m_loc = -INFINITY;
-#pragma unroll
-      for (int kt = 0; kt < T::kKeyTiles; ++kt)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) m_loc = fmaxf(m_loc, s[qt][kt][e]);
-      m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
-      const float m_new = fmaxf(m_run[qt], m_loc);
-      const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
-      float psum = 0.0f;
-#pragma unroll
-      for (int kt = 0; kt < T::kKeyTiles; ++kt) {
-#pragma unroll
-        for (int e = 0; e < 16; e += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(s[qt][kt][e] - m_use);
-          const float p1 = __builtin_amdgcn_exp2f(s[qt][kt][e + 1] - m_use);
-          psum += p0 + p1;
-          p[qt][kt][e / 2] = pack_bf16(p0, p1);
-        }
-      }
-      l_run[qt] = l_run[qt] * alpha + psum;
-      m_run[qt] = m_new;
-#pragma unroll
-      for (int i = 0; i < T::kDTiles; ++i)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc_o[qt][i][e] *= alpha;
-    }
-
-    store_tile(Vs, T::kPitchV);
-    __syncthreads();  // V tile visible; every wave is done reading Ks
-
-    const bool more = (t + 1) < n_tiles;
-    if (more) load_tile(Kb, kv0 + BC);
-
-    // ---- O^T += V^T . P^T ----
-#pragma unroll
-    for (int kt = 0; kt < T::kKeyTiles; ++kt) {
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const uint16_t *vp = Vs + (kt * 32 + 16 * b) * T::kPitchV + vtr_off;
-#pragma unroll
-        for (int i = 0; i < T::kDTiles; ++i) {
-          const bf16x4_v lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-              (KCG_LDS_BF16X4 *)(vp + 32 * i));
-          const bf16x4_v hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-              (KCG_LDS_BF16X4 *)(vp + 8 * T::kPitchV + 32 * i));
-          const bf16x8_v vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-          for (int qt = 0; qt < QT; ++qt) {
-            const u32x4_t pw = {p[qt][kt][4 * b], p[qt][kt][4 * b + 1], p[qt][kt][4 * b + 2],
-                                p[qt][kt][4 * b + 3]};
-            acc_o[qt][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                vf, __builtin_bit_cast(bf16x8_v, pw), acc_o[qt][i], 0, 0, 0);
-          }
-        }
-      }
-    }
-
-    if (more) store_tile(Ks, T::kPitchK);
-    __syncthreads();  // next K tile visible; every wave is done reading Vs
-  }
-
-  // ---- normalise and store: lane holds O[qrow][32*i + 8*g + 4*half + 0..3] ----
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    const int qrow = wq0 + 32 * qt + r32;
-    const float l_tot = l_run[qt] + __shfl_xor(l_run[qt], 32);
-    const float inv = 1.0f / l_tot;
-    if (qrow < S) {
-      const int64_t off = base + static_cast<int64_t>(qrow) * D + 4 * half;
-#pragma unroll
-      for (int i = 0; i < T::kDTiles; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const float v0 = acc_o[qt][i][4 * g + 0] * inv;
-          const float v1 = acc_o[qt][i][4 * g + 1] * inv;
-          const float v2 = acc_o[qt][i][4 * g + 2] * inv;
-          const float v3 = acc_o[qt][i][4 * g + 3] * inv;
-          if (OUT_BF16) {
-            u32x2_t w = {pack_bf16(v0, v1), pack_bf16(v2, v3)};
-            *reinterpret_cast<u32x2_t *>(static_cast<uint16_t *>(O) + off + 32 * i + 8 * g) = w;
-          } else {
-            float4_t w = {v0, v1, v2, v3};
-            *reinterpret_cast<float4_t *>(static_cast<float *>(O) + off + 32 * i + 8 * g) = w;
-          }
-        }
     }
   }
 }
 
-template <int D, int BC, int QT>
+template <int D, int BC, int QT, bool POS>
 static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O,
                             int o_dtype, int B, int H, int S, float scale, int causal,
                             hipStream_t stream, kcg_launch_info *info) {
   using T = FmhaBf16Tile<D, BC, QT>;
   const int64_t q_blocks = (static_cast<int64_t>(S) + T::kBr - 1) / T::kBr;
-  const int64_t blocks = q_blocks * B * H;
+  const int64_t q_items = causal ? (q_blocks + 1) / 2 : q_blocks;
+  const int64_t blocks = q_items * B * H;
   if (blocks > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
   if (info) {
     info->grid[0] = static_cast<int>(blocks);
@@ -308,24 +439,25 @@ static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t
     info->lds_bytes = T::kLdsBytes;
     info->waves_per_block = 4;
     snprintf(info->kernel, sizeof info->kernel, "fmha_bf16_d%d_br%d_bc%d%s", D, T::kBr, BC,
-             causal ? "_causal" : "");
+             causal ? "_causal_paired" : "");
     return KCG_OK;
   }
   const float scale_log2e = scale * 1.4426950408889634f;
-#define KCG_LAUNCH(CAUSAL_, OBF_)                                                                 \
+#define KCG_LAUNCH(CAUSAL_, OBF_, POS_)                                                                 \
   do {                                                                                            \
-    auto kern = fmha_bf16_kernel<D, BC, QT, CAUSAL_, OBF_>;                                       \
+    auto kern = fmha_bf16_kernel<D, BC, QT, CAUSAL_, OBF_, POS_>;                                       \
     if (!allow_lds(kern, T::kLdsBytes)) return KCG_ERR_LAUNCH;                                    \
     return launch(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads), T::kLdsBytes,     \
-                  stream, Q, K, V, O, S, static_cast<int>(q_blocks), scale_log2e);                \
+                  stream, Q, K, V, O, S, static_cast<int>(q_blocks), static_cast<int>(q_items),   \
+                  scale_log2e);                                                                   \
   } while (0)
   const bool obf = o_dtype == KCG_BF16;
   if (causal) {
-    if (obf) KCG_LAUNCH(true, true);
-    else KCG_LAUNCH(true, false);
+    if (obf) KCG_LAUNCH(true, true, POS);
+    else KCG_LAUNCH(true, false, POS);
   } else {
-    if (obf) KCG_LAUNCH(false, true);
-    else KCG_LAUNCH(false, false);
+    if (obf) KCG_LAUNCH(false, true, POS);
+    else KCG_LAUNCH(false, false, POS);
   }
 #undef KCG_LAUNCH
 }
@@ -339,20 +471,23 @@ int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, 
     if (sched->bc) bc = sched->bc;
   }
   if (bc != 64) return KCG_ERR_BAD_SCHEDULE;
-  if (D == 128) {
-    if (br == 128)
-      return launch_fmha_bf16<128, 64, 1>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, info);
-    if (br == 256)
-      return launch_fmha_bf16<128, 64, 2>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, info);
-    return KCG_ERR_BAD_SCHEDULE;
+  if (br != 128 && br != 256) return KCG_ERR_BAD_SCHEDULE;
+  // scale <= 0 takes the general softmax path, built for the 128-row block only
+  const bool pos = scale > 0.0f;
+#define KCG_PICK(D_)                                                                              \
+  if (D == D_) {                                                                                  \
+    if (!pos)                                                                                     \
+      return launch_fmha_bf16<D_, 64, 1, false>(Q, K, V, O, o_dtype, B, H, S, scale, causal,      \
+                                                stream, info);                                    \
+    if (br == 128)                                                                                \
+      return launch_fmha_bf16<D_, 64, 1, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal,       \
+                                               stream, info);                                     \
+    return launch_fmha_bf16<D_, 64, 2, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, \
+                                             info);                                               \
   }
-  if (D == 64) {
-    if (br == 128)
-      return launch_fmha_bf16<64, 64, 1>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, info);
-    if (br == 256)
-      return launch_fmha_bf16<64, 64, 2>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, info);
-    return KCG_ERR_BAD_SCHEDULE;
-  }
+  KCG_PICK(128)
+  KCG_PICK(64)
+#undef KCG_PICK
   return KCG_ERR_UNSUPPORTED_SHAPE;
 }
 
