@@ -7,8 +7,8 @@
 // Softmax -> BatchedMatmul(P, V) (test/test.cc:88-90), with the optional scale
 // and causal mask.
 //
-// Work split: 4 waves per workgroup, QT*32 query rows per wave (Br = 128*QT),
-// K/V swept in tiles of BC = 64 rows.
+// Work split: WAVES (4 or 8) waves per workgroup, 32 query rows per wave
+// (Br = 128 or 256), K/V swept in tiles of BC = 64 rows.
 //
 //  * S^T = K . Q^T: A operand = K rows from LDS (one ds_read_b128 = 8 bf16 of d
 //    per lane), B operand = Q, held in registers for the whole sweep.  Lane
@@ -58,22 +58,26 @@ typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 #define KCG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define KCG_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
-template <int D, int BC, int QT>
+template <int D, int BC, int QT, int WAVES>
 struct FmhaBf16Tile {
-  static constexpr int kThreads = 256;
-  static constexpr int kBr = 128 * QT;
+  static constexpr int kThreads = 64 * WAVES;
+  static constexpr int kBr = 32 * QT * WAVES;
   static constexpr int kWaveRows = 32 * QT;
   static constexpr int kCpr = D / 8;            // 16-byte chunks per row
   static constexpr int kRowsPer256 = 16 / kCpr;  // rows that share one 256-byte bank window
   static constexpr int kRpi = 64 / kCpr;         // rows filled by one wave-wide direct load
-  static constexpr int kIpw = BC / kRpi / 4;     // direct loads per wave per tile
+  static constexpr int kIpw = BC / kRpi / WAVES;  // direct loads per wave per tile
   static constexpr int kTile = BC * D;           // elements per K (or V) buffer, unpadded
-  static constexpr int kLdsBytes = 2 * 2 * kTile * 2;  // K and V, double-buffered
+  // K/V tile buffers: a ring of 2 (tile t+1 streams in while tile t is consumed).  A ring
+  // of 3 with loads two tiles ahead was measured slower for the 8-wave workgroup.
+  static constexpr int kRing = 2;
+  static constexpr int kAheadTiles = kRing - 1;
+  static constexpr int kLdsBytes = kRing * 2 * kTile * 2;
   static constexpr int kKeyTiles = BC / 32;
   static constexpr int kDTiles = D / 32;
   static constexpr int kDSteps = D / 16;
   static_assert(D == 64 || D == 128, "head dim");
-  static_assert(BC % (4 * kRpi) == 0 && BC % 32 == 0, "tile extents");
+  static_assert(BC % (WAVES * kRpi) == 0 && BC % 32 == 0, "tile extents");
   // chunk-index swizzles (see the file header)
   __host__ __device__ static constexpr int fk(int row) { return (row / kRowsPer256) % kCpr; }
   __host__ __device__ static constexpr int fv(int row) { return 4 * ((row / kRowsPer256) & (kCpr / 4 - 1)); }
@@ -100,14 +104,14 @@ constexpr float kTau = 8.0f;
 
 // POS_SCALE: scale > 0, so exp2(s * c - m) is one FMA and the row maximum can be
 // taken on the raw products.  The general variant scales first.
-template <int D, int BC, int QT, bool CAUSAL, bool OUT_BF16, bool POS_SCALE>
-__global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
+template <int D, int BC, int QT, int WAVES, bool CAUSAL, bool OUT_BF16, bool POS_SCALE>
+__global__ __launch_bounds__(64 * WAVES, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     void *__restrict__ O, int S, int q_blocks, int q_items, float scale_log2e) {
-  using T = FmhaBf16Tile<D, BC, QT>;
+  using T = FmhaBf16Tile<D, BC, QT, WAVES>;
   extern __shared__ __align__(16) uint16_t lds16[];
-  uint16_t *Ks = lds16;                  // [2][BC][D], chunk-swizzled
-  uint16_t *Vs = lds16 + 2 * T::kTile;   // [2][BC][D], chunk-swizzled
+  uint16_t *Ks = lds16;                  // [kRing][BC][D], chunk-swizzled
+  uint16_t *Vs = lds16 + T::kRing * T::kTile;   // [kRing][BC][D], chunk-swizzled
 
   // Every XCD walks a contiguous range of (head, work item) ids, head-major, so
   // the K/V of a head are fetched into one XCD's L2 only.  Causal: a work item is
@@ -137,41 +141,53 @@ __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
   const int ld_row0 = wave * T::kIpw * T::kRpi;
   const int ld_lrow = lane / T::kCpr;
   const int ld_pos = lane % T::kCpr;
-  int goff_k[T::kIpw], goff_v[T::kIpw];  // element offsets inside a tile, per instruction
+  unsigned goff_k[T::kIpw], goff_v[T::kIpw];  // byte offsets inside a tile, per instruction
 #pragma unroll
   for (int j = 0; j < T::kIpw; ++j) {
     const int row = ld_row0 + j * T::kRpi + ld_lrow;
-    goff_k[j] = row * D + (ld_pos ^ T::fk(row)) * 8;
-    goff_v[j] = row * D + (ld_pos ^ T::fv(row)) * 8;
+    goff_k[j] = static_cast<unsigned>(row * D + (ld_pos ^ T::fk(row)) * 8) * 2u;
+    goff_v[j] = static_cast<unsigned>(row * D + (ld_pos ^ T::fv(row)) * 8) * 2u;
   }
-  auto load_tiles = [&](int kv0, int buf) {
-    const uint16_t *kg = Kb + static_cast<int64_t>(kv0) * D;
-    const uint16_t *vg = Vb + static_cast<int64_t>(kv0) * D;
+  // One direct load (K for even `which`, V for odd) of the tile at kv0 into buffer `buf`:
+  // uniform 64-bit tile base + per-lane 32-bit byte offset.
+  auto load_one = [&](int kv0, int buf, int which) {
+    const int j = which >> 1;
+    const char *g = reinterpret_cast<const char *>(((which & 1) ? Vb : Kb) + static_cast<int64_t>(kv0) * D);
+    uint16_t *l = ((which & 1) ? Vs : Ks) + buf * T::kTile + (ld_row0 + j * T::kRpi) * D;
+    const unsigned off = (which & 1) ? goff_v[j] : goff_k[j];
+    __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(g + off), KCG_LDS_PTR(l), 16, 0, 0);
+  };
+  // Ragged last tile: rows at and beyond S are zero-filled, through registers.
+  auto load_tiles_ragged = [&](int kv0, int buf) {
+    const char *kg = reinterpret_cast<const char *>(Kb + static_cast<int64_t>(kv0) * D);
+    const char *vg = reinterpret_cast<const char *>(Vb + static_cast<int64_t>(kv0) * D);
     uint16_t *kl = Ks + buf * T::kTile + ld_row0 * D;
     uint16_t *vl = Vs + buf * T::kTile + ld_row0 * D;
+#pragma unroll
+    for (int j = 0; j < T::kIpw; ++j) {
+      const int row = ld_row0 + j * T::kRpi + ld_lrow;
+      const bool ok = kv0 + row < S;
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+      const u32x4_t kvq = ok ? *reinterpret_cast<const u32x4_t *>(kg + goff_k[j]) : z;
+      const u32x4_t vvq = ok ? *reinterpret_cast<const u32x4_t *>(vg + goff_v[j]) : z;
+      *reinterpret_cast<u32x4_t *>(kl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = kvq;
+      *reinterpret_cast<u32x4_t *>(vl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = vvq;
+    }
+  };
+  auto load_tiles = [&](int kv0, int buf) {
     if (kv0 + BC <= S) {
 #pragma unroll
-      for (int j = 0; j < T::kIpw; ++j) {
-        __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(kg + goff_k[j]), KCG_LDS_PTR(kl + j * T::kRpi * D), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(vg + goff_v[j]), KCG_LDS_PTR(vl + j * T::kRpi * D), 16, 0, 0);
-      }
+      for (int w = 0; w < 2 * T::kIpw; ++w) load_one(kv0, buf, w);
     } else {
-      // ragged last tile: rows at and beyond S are zero-filled, through registers
-#pragma unroll
-      for (int j = 0; j < T::kIpw; ++j) {
-        const int row = ld_row0 + j * T::kRpi + ld_lrow;
-        const bool ok = kv0 + row < S;
-        const u32x4_t z = {0u, 0u, 0u, 0u};
-        const u32x4_t kvq = ok ? *reinterpret_cast<const u32x4_t *>(kg + goff_k[j]) : z;
-        const u32x4_t vvq = ok ? *reinterpret_cast<const u32x4_t *>(vg + goff_v[j]) : z;
-        *reinterpret_cast<u32x4_t *>(kl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = kvq;
-        *reinterpret_cast<u32x4_t *>(vl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = vvq;
-      }
+      load_tiles_ragged(kv0, buf);
     }
   };
   // Every wave waits for its own direct loads; the barrier then publishes all of them.
-  auto tiles_ready = [&]() {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // `in_flight` = direct loads this wave may leave outstanding (those of tiles further
+  // ahead than the next one).
+  auto tiles_ready = [&](bool keep_newest) {
+    if (keep_newest) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * T::kIpw) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   };
 
@@ -189,6 +205,8 @@ __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
 
 #pragma unroll 1
   for (int pass = 0; pass < npass; ++pass) {
+    // the long block goes first: the long sweeps of a head's workgroups then start together
+    // and share each K/V tile in L2 (short-first was measured to fetch 26% more)
     const int qb = CAUSAL ? (pass == 0 ? hi_block : item) : item;
     const int q0 = qb * T::kBr;
     const int wq0 = q0 + wave * T::kWaveRows;  // first query row of this wave
@@ -225,15 +243,23 @@ __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
     const int n_tiles = (kv_end + BC - 1) / BC;
 
     load_tiles(0, 0);
-    tiles_ready();
+    if (T::kAheadTiles > 1 && n_tiles > 1) load_tiles(BC, 1);
+    tiles_ready(false);
 
     for (int t = 0; t < n_tiles; ++t) {
       const int kv0 = t * BC;
-      const int cur = t & 1;
-      if (t + 1 < n_tiles) load_tiles(kv0 + BC, cur ^ 1);  // streams in while this tile is computed
+      const int cur = t % T::kRing;
+      const int nxt = (t + T::kAheadTiles) % T::kRing;  // buffer of the tile fetched in this step
+      // the next tile streams in while this one is computed; when it is a full tile its
+      // direct loads are issued one per d-step, between the MFMAs of S = K.Q^T
+      const bool more = t + T::kAheadTiles < n_tiles;
+      const int kv_nxt = kv0 + T::kAheadTiles * BC;
+      const bool spread = more && (kv_nxt + BC <= S);
+      if (more && !spread) load_tiles(kv_nxt, nxt);
 
       // A wave whose last query precedes the tile has nothing to add (causal).
       const bool wave_active = !CAUSAL || (kv0 <= wq0 + T::kWaveRows - 1);
+      if (spread && !wave_active) load_tiles(kv_nxt, nxt);
       if (wave_active) {
         const uint16_t *ks = Ks + cur * T::kTile + k_row_off;
         const uint16_t *vs = Vs + cur * T::kTile + v_row_off;
@@ -261,6 +287,7 @@ __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
 #pragma unroll
           for (int ds = 0; ds < T::kDSteps; ++ds) {
             if (ds + kAhead < T::kDSteps) fetch(ds + kAhead);
+            if (ds < 2 * T::kIpw && spread) load_one(kv_nxt, nxt, ds);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kt = 0; kt < T::kKeyTiles; ++kt)
@@ -390,7 +417,9 @@ __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
         }
       }
 
-      tiles_ready();  // next tiles visible; every wave is done with the current buffers
+      // the next tile is complete and visible after this; with a ring of 3 the loads of
+      // the tile after it (issued in this step, when direct) stay in flight
+      tiles_ready(T::kAheadTiles > 1 && spread);
     }
 
     // ---- normalise and store: lane holds O[qrow][32*i + 8*g + 4*half + 0..3] ----
@@ -422,11 +451,11 @@ __global__ __launch_bounds__(256, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
   }
 }
 
-template <int D, int BC, int QT, bool POS>
+template <int D, int BC, int QT, int WAVES, bool POS>
 static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O,
                             int o_dtype, int B, int H, int S, float scale, int causal,
                             hipStream_t stream, kcg_launch_info *info) {
-  using T = FmhaBf16Tile<D, BC, QT>;
+  using T = FmhaBf16Tile<D, BC, QT, WAVES>;
   const int64_t q_blocks = (static_cast<int64_t>(S) + T::kBr - 1) / T::kBr;
   const int64_t q_items = causal ? (q_blocks + 1) / 2 : q_blocks;
   const int64_t blocks = q_items * B * H;
@@ -437,7 +466,7 @@ static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t
     info->block[0] = T::kThreads;
     info->block[1] = info->block[2] = 1;
     info->lds_bytes = T::kLdsBytes;
-    info->waves_per_block = 4;
+    info->waves_per_block = WAVES;
     snprintf(info->kernel, sizeof info->kernel, "fmha_bf16_d%d_br%d_bc%d%s", D, T::kBr, BC,
              causal ? "_causal_paired" : "");
     return KCG_OK;
@@ -445,7 +474,7 @@ static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t
   const float scale_log2e = scale * 1.4426950408889634f;
 #define KCG_LAUNCH(CAUSAL_, OBF_, POS_)                                                                 \
   do {                                                                                            \
-    auto kern = fmha_bf16_kernel<D, BC, QT, CAUSAL_, OBF_, POS_>;                                       \
+    auto kern = fmha_bf16_kernel<D, BC, QT, WAVES, CAUSAL_, OBF_, POS_>;                                       \
     if (!allow_lds(kern, T::kLdsBytes)) return KCG_ERR_LAUNCH;                                    \
     return launch(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads), T::kLdsBytes,     \
                   stream, Q, K, V, O, S, static_cast<int>(q_blocks), static_cast<int>(q_items),   \
@@ -465,7 +494,9 @@ static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t
 int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O,
                        int o_dtype, int B, int H, int S, int D, float scale, int causal,
                        const kcg_fmha_sched *sched, hipStream_t stream, kcg_launch_info *info) {
-  int br = 128, bc = 64;
+  // default: 8 waves (256 query rows) share each K/V tile once the sequence is long
+  // enough to keep every CU busy with such workgroups
+  int br = S >= 2048 ? 256 : 128, bc = 64;
   if (sched) {
     if (sched->br) br = sched->br;
     if (sched->bc) bc = sched->bc;
@@ -477,12 +508,12 @@ int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, 
 #define KCG_PICK(D_)                                                                              \
   if (D == D_) {                                                                                  \
     if (!pos)                                                                                     \
-      return launch_fmha_bf16<D_, 64, 1, false>(Q, K, V, O, o_dtype, B, H, S, scale, causal,      \
+      return launch_fmha_bf16<D_, 64, 1, 4, false>(Q, K, V, O, o_dtype, B, H, S, scale, causal,      \
                                                 stream, info);                                    \
     if (br == 128)                                                                                \
-      return launch_fmha_bf16<D_, 64, 1, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal,       \
+      return launch_fmha_bf16<D_, 64, 1, 4, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal,       \
                                                stream, info);                                     \
-    return launch_fmha_bf16<D_, 64, 2, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, \
+    return launch_fmha_bf16<D_, 64, 1, 8, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, \
                                              info);                                               \
   }
   KCG_PICK(128)

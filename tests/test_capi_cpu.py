@@ -78,8 +78,14 @@ def test_launch_geometry_queries():
     assert L.kcg_gemm_f32_query(4096, 4096, 4096, None, ctypes.byref(info)) == 0
     assert info.grid[0] * 256 * 128 == 4096 * 4096 and info.lds_bytes <= 160 * 1024
     assert L.kcg_gemm_f32_query(100, 100, 100, None, None) == 1
+    # bf16 causal, S = 4096: 256-row query blocks run in pairs (n-1-i, i) -> 8 work items per head
     assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 1, None, ctypes.byref(info)) == 0
-    assert info.grid[0] % (4 * 32) == 0 and info.block[0] == 256
+    assert info.grid[0] == 4 * 32 * 8 and info.block[0] == 512 and info.waves_per_block == 8
+    s128 = lib.FmhaSched(br=128, bc=64)
+    assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 1, ctypes.byref(s128), ctypes.byref(info)) == 0
+    assert info.grid[0] == 4 * 32 * 16 and info.block[0] == 256
+    assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 0, ctypes.byref(s128), ctypes.byref(info)) == 0
+    assert info.grid[0] == 4 * 32 * 32 and info.lds_bytes == 2 * 2 * 64 * 128 * 2
     assert L.kcg_fmha_query(0, 1, 32, 2048, 128, 0, None, ctypes.byref(info)) == 0
     assert info.grid[0] == 32 * 2048 // 128
     assert L.kcg_fmha_query(7, 1, 1, 128, 128, 0, None, ctypes.byref(info)) == 5

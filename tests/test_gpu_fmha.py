@@ -180,3 +180,35 @@ def test_errors(dev):
     q = torch.zeros(1, 1, 64, 64, device=dev)
     with pytest.raises(ValueError):
         ops.fmha(q, q[:, :, :32], q)
+
+
+@pytest.mark.parametrize("scale", [-0.2, 0.0])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_non_positive_scale(oracle, dev, scale, dtype):
+    """scale <= 0 takes the kernels' general softmax path (the fast path needs scale > 0)."""
+    from kernelcodegen_amd import ops
+    shape = (1, 2, 200, 128)
+    Q, K, V = (inputs.normal(shape, 205, i) for i in range(3))
+    if dtype == "bf16":
+        Qb, Kb, Vb = (inputs.to_bf16_bits(t) for t in (Q, K, V))
+        ref = oracle.fmha(Qb, Kb, Vb, scale=scale, causal=True, stable=True)
+        O = ops.fmha(*(_gpu_bf16(t, dev) for t in (Qb, Kb, Vb)), scale=scale, causal=True)
+        assert max(rel_err(O.float().cpu().numpy(), ref)) < TOL_BF16
+    else:
+        ref = oracle.fmha(Q, K, V, scale=scale, causal=True, stable=True)
+        O = ops.fmha(*(_gpu(t, dev) for t in (Q, K, V)), scale=scale, causal=True)
+        assert max(rel_err(O.cpu().numpy(), ref)) < TOL_F32
+
+
+def test_bf16_default_schedule_and_large_logits(oracle, dev):
+    """Default schedule (8-wave workgroups from S = 2048 on) and a logit scale large
+    enough that the running maximum keeps growing, which exercises the lazy rescale."""
+    import torch
+    from kernelcodegen_amd import ops
+    shape = (1, 2, 2048 + 70, 128)
+    Q, K, V = (inputs.to_bf16_bits(inputs.normal(shape, 206, i)) for i in range(3))
+    tq, tk, tv = (_gpu_bf16(t, dev) for t in (Q, K, V))
+    for scale, causal in [(128 ** -0.5, True), (0.75, False), (0.75, True)]:
+        ref = oracle.fmha(Q, K, V, scale=scale, causal=causal, stable=True, rows=(1990, 2118))
+        O = ops.fmha(tq, tk, tv, scale=scale, causal=causal, out_dtype=torch.float32)
+        assert max(rel_err(O[:, :, 1990:2118].cpu().numpy(), ref)) < TOL_BF16
