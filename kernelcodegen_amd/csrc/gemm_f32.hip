@@ -253,7 +253,31 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
 static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
                          int epilogue, const kcg_gemm_sched *s, hipStream_t stream,
                          kcg_launch_info *info) {
+  // Default tile by problem size.  Workgroups are spread over 256 CUs and the CU
+  // with the most workgroups sets the run time, so a tile is scored by
+  //   (its measured large-problem efficiency) x (tiles / (256 * max tiles per CU));
+  // small or awkwardly sized problems thereby get smaller tiles instead of leaving
+  // most of the chip idle (the reference's fixed 128x128 tile does the latter).
   kcg_gemm_sched d = {256, 128, 16, 8, 64, 64, 4, 64};
+  if (!s || (s->block_m == 0 && s->block_n == 0)) {
+    struct Cand {
+      int bm, bn, bk, wm, wn;
+      double eff;
+    };
+    const Cand cands[] = {{256, 128, 16, 64, 64, 0.88}, {128, 128, 16, 64, 64, 0.86}, {64, 64, 32, 32, 32, 0.77}};
+    double best = -1.0;
+    for (const Cand &c : cands) {
+      const double tiles = static_cast<double>((M + c.bm - 1) / c.bm) * static_cast<double>((N + c.bn - 1) / c.bn);
+      const double per_cu = static_cast<double>((static_cast<int64_t>(tiles) + kNumCu - 1) / kNumCu);
+      // padding waste of ragged edges counts against a large tile too
+      const double useful = (static_cast<double>(M) * N) / (tiles * c.bm * c.bn);
+      const double score = c.eff * useful * tiles / (per_cu * kNumCu);
+      if (score > best) {
+        best = score;
+        d = {c.bm, c.bn, c.bk, 8, c.wm, c.wn, 4, 64};
+      }
+    }
+  }
   if (s) {
     if (s->block_m) d.block_m = s->block_m;
     if (s->block_n) d.block_n = s->block_n;

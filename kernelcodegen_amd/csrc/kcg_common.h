@@ -19,6 +19,7 @@ typedef short bf16x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned short u16x8_t __attribute__((ext_vector_type(8)));
 
 constexpr int kWaveSize = 64;
+constexpr int kNumCu = 256;  // MI355X compute units
 constexpr int kNumXcd = 8;  // MI355X: 8 XCDs, workgroups are dealt to them round-robin
 
 // Workgroup id -> logical tile id such that every XCD (which owns a private L2)
