@@ -91,16 +91,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   float4_t ra[T::kLoadsA];
   float4_t rb[T::kLoadsB];
 
-  auto load_global = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < T::kLoadsA; ++i) {
-      const int idx = tid + i * T::kThreads;
+  // Transfer g of a K slice: g < kLoadsA moves one float4 of A per thread, the
+  // rest one float4 of B.  load_one: global -> registers; store_one: registers -> LDS.
+  constexpr int kTransfers = T::kLoadsA + T::kLoadsB;
+  auto load_one = [&](int g, int k0) {
+    if (g < T::kLoadsA) {
+      const int idx = tid + g * T::kThreads;
       const int row = idx / (BK / 4);
       const int c4 = idx % (BK / 4);
       const int64_t gr = m0 + row;
       const int gk = k0 + c4 * 4;
       if (FULL) {
-        ra[i] = *reinterpret_cast<const float4_t *>(A + gr * K + gk);
+        ra[g] = *reinterpret_cast<const float4_t *>(A + gr * K + gk);
       } else {
         float4_t v = {0.f, 0.f, 0.f, 0.f};
         if (gr < M) {
@@ -109,11 +111,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
           for (int e = 0; e < 4; ++e)
             if (gk + e < K) v[e] = p[gk + e];
         }
-        ra[i] = v;
+        ra[g] = v;
       }
-    }
-#pragma unroll
-    for (int i = 0; i < T::kLoadsB; ++i) {
+    } else {
+      const int i = g - T::kLoadsA;
       const int idx = tid + i * T::kThreads;
       const int row = idx / (BN / 4);
       const int c4 = idx % (BN / 4);
@@ -133,60 +134,106 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       }
     }
   };
-
-  auto store_lds = [&](int buf) {
-    float *as = As + buf * T::kFloatsA;
-    float *bs = Bs + buf * T::kFloatsB;
-#pragma unroll
-    for (int i = 0; i < T::kLoadsA; ++i) {
-      const int idx = tid + i * T::kThreads;
+  auto store_one = [&](int g, int buf) {
+    if (g < T::kLoadsA) {
+      const int idx = tid + g * T::kThreads;
       const int row = idx / (BK / 4);
       const int c4 = idx % (BK / 4);
-      *reinterpret_cast<float4_t *>(as + row * T::kPitchA + c4 * 4) = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < T::kLoadsB; ++i) {
+      *reinterpret_cast<float4_t *>(As + buf * T::kFloatsA + row * T::kPitchA + c4 * 4) = ra[g];
+    } else {
+      const int i = g - T::kLoadsA;
       const int idx = tid + i * T::kThreads;
       const int row = idx / (BN / 4);
       const int c4 = idx % (BN / 4);
-      *reinterpret_cast<float4_t *>(bs + row * T::kPitchB + c4 * 4) = rb[i];
+      *reinterpret_cast<float4_t *>(Bs + buf * T::kFloatsB + row * T::kPitchB + c4 * 4) = rb[i];
     }
   };
-
-  auto compute = [&](int buf) {
-    const float *as = As + buf * T::kFloatsA + (wm * T::kWaveM + r32) * T::kPitchA + 4 * half;
-    const float *bs = Bs + buf * T::kFloatsB + (4 * half) * T::kPitchB + wn * T::kWaveN + r32;
-#pragma unroll
-    for (int kk = 0; kk < BK / 8; ++kk) {
-      float4_t a[T::kTilesM];
-#pragma unroll
-      for (int i = 0; i < T::kTilesM; ++i)
-        a[i] = *reinterpret_cast<const float4_t *>(as + i * 32 * T::kPitchA + kk * 8);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float b[T::kTilesN];
-#pragma unroll
-        for (int n = 0; n < T::kTilesN; ++n) b[n] = bs[(kk * 8 + j) * T::kPitchB + n * 32];
-#pragma unroll
-        for (int i = 0; i < T::kTilesM; ++i)
-#pragma unroll
-          for (int n = 0; n < T::kTilesN; ++n)
-            acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][j], b[n], acc[i][n], 0, 0, 0);
-      }
-    }
-  };
+  // ---- main loop --------------------------------------------------------
+  // One K slice is consumed in kSteps steps of kTilesM*kTilesN MFMAs; step s
+  // takes k = 8*(s/4) + 4*half + s%4.  The operands of step s+1 are read from
+  // LDS before the MFMAs of step s are issued, so the LDS latency sits under
+  // the matrix pipe.  Slice kt+1, which arrived in registers during slice
+  // kt-1, is written to the other LDS buffer at the top of slice kt and the
+  // registers are refilled with slice kt+2.  The one barrier per slice comes
+  // before the LAST step of slice kt: at that point every wave holds its last
+  // operands of slice kt in registers, so the barrier both publishes slice
+  // kt+1 and releases buffer `cur` for the writes of the next iteration, and
+  // the first operands of slice kt+1 are read while the last MFMAs of slice kt
+  // still run.
+  constexpr int kSteps = BK / 2;
+  const float *a_base = As + (wm * T::kWaveM + r32) * T::kPitchA + 4 * half;
+  const float *b_base = Bs + (4 * half) * T::kPitchB + wn * T::kWaveN + r32;
+  float4_t fa[2][T::kTilesM];
+  float fb[2][T::kTilesN];
+  float4_t na[T::kTilesM];
+  float nb[T::kTilesN];
 
   const int ktiles = (K + BK - 1) / BK;
-  load_global(0);
-  store_lds(0);
+#pragma unroll
+  for (int g = 0; g < kTransfers; ++g) load_one(g, 0);
+#pragma unroll
+  for (int g = 0; g < kTransfers; ++g) store_one(g, 0);
+  if (ktiles > 1) {
+#pragma unroll
+    for (int g = 0; g < kTransfers; ++g) load_one(g, BK);
+  }
   __syncthreads();
+#pragma unroll
+  for (int i = 0; i < T::kTilesM; ++i)
+    na[i] = *reinterpret_cast<const float4_t *>(a_base + i * 32 * T::kPitchA);
+#pragma unroll
+  for (int n = 0; n < T::kTilesN; ++n) nb[n] = b_base[n * 32];
+
   for (int kt = 0; kt < ktiles; ++kt) {
     const int cur = kt & 1;
-    const bool more = (kt + 1) < ktiles;
-    if (more) load_global((kt + 1) * BK);
-    compute(cur);
-    if (more) store_lds(cur ^ 1);
-    __syncthreads();
+    const float *as = a_base + cur * T::kFloatsA;
+    const float *bs = b_base + cur * T::kFloatsB;
+#pragma unroll
+    for (int i = 0; i < T::kTilesM; ++i) fa[0][i] = na[i];
+#pragma unroll
+    for (int n = 0; n < T::kTilesN; ++n) fb[0][n] = nb[n];
+    if (kt + 1 < ktiles) {
+#pragma unroll
+      for (int g = 0; g < kTransfers; ++g) store_one(g, cur ^ 1);
+    }
+    if (kt + 2 < ktiles) {
+#pragma unroll
+      for (int g = 0; g < kTransfers; ++g) load_one(g, (kt + 2) * BK);
+    }
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      if (s + 1 < kSteps) {
+        const int s1 = s + 1;
+        if (s1 % 4 == 0) {
+#pragma unroll
+          for (int i = 0; i < T::kTilesM; ++i)
+            fa[(s1 / 4) & 1][i] =
+                *reinterpret_cast<const float4_t *>(as + i * 32 * T::kPitchA + (s1 / 4) * 8);
+        }
+#pragma unroll
+        for (int n = 0; n < T::kTilesN; ++n)
+          fb[s1 & 1][n] = bs[((s1 / 4) * 8 + s1 % 4) * T::kPitchB + n * 32];
+      } else {
+        __syncthreads();
+        if (kt + 1 < ktiles) {
+          const float *as1 = a_base + (cur ^ 1) * T::kFloatsA;
+          const float *bs1 = b_base + (cur ^ 1) * T::kFloatsB;
+#pragma unroll
+          for (int i = 0; i < T::kTilesM; ++i)
+            na[i] = *reinterpret_cast<const float4_t *>(as1 + i * 32 * T::kPitchA);
+#pragma unroll
+          for (int n = 0; n < T::kTilesN; ++n) nb[n] = bs1[n * 32];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < T::kTilesM; ++i)
+#pragma unroll
+        for (int n = 0; n < T::kTilesN; ++n)
+          acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[(s / 4) & 1][i][s % 4], fb[s & 1][n],
+                                                           acc[i][n], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 
   // ---- epilogue + writeback: per store, lanes 0-31 and 32-63 each cover one
@@ -202,6 +249,266 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
         float v = acc[i][n][e];
         if (RELU) v = relu_maxf(v);
         if (FULL || (row < M && col < N)) C[static_cast<int64_t>(row) * N + col] = v;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Full-tile kernel with direct global->LDS loads.
+//
+// For problems whose sizes divide the tile the K slices never pass through
+// registers: global_load_lds_dwordx4 writes lane l's 16 bytes at (wave-uniform
+// LDS base) + 16*l, so each instruction fills a 1 KiB run of LDS and each lane
+// is free to fetch whichever global chunk belongs there.  Rows inside a run
+// cannot be padded; bank conflicts are avoided like this instead:
+//   As[stage][BM][BK]   16-byte chunk c of row m is stored at chunk c ^ fa(m),
+//                       fa(m) = ((m / rows-per-128B) % chunks-per-row) ^ ((m/8) & 1):
+//                       any 8 consecutive rows fill a 128-byte window and any 16
+//                       a 256-byte window without sharing a slot, so the
+//                       ds_read_b128 of one chunk column is conflict free.
+//   Bs[stage][BK][BN]   rows as in global memory, 1 KiB runs (256/BN rows each)
+//                       spaced 1 KiB + 8192/BN bytes apart, which puts rows k and
+//                       k+4 (read together by the two halves of a wave) 128 bytes
+//                       apart modulo 256.
+// Three LDS stages: slice kt+2 is requested at the top of slice kt and has two
+// slices of MFMA time to arrive; a wave only waits for its own loads of slice
+// kt+1 (vmcnt) right before the barrier that publishes them.
+#define KCG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define KCG_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+struct GemmDlTile {
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * kWaveSize;
+  static constexpr int kWaveM = BM / WAVES_M;
+  static constexpr int kWaveN = BN / WAVES_N;
+  static constexpr int kTilesM = kWaveM / 32;
+  static constexpr int kTilesN = kWaveN / 32;
+  static constexpr int kCprA = BK / 4;        // 16-byte chunks per A row
+  static constexpr int kRp128A = 8 / kCprA;   // A rows per 128 bytes
+  static constexpr int kFloatsA = BM * BK;
+  static constexpr int kRowsPerRunB = 256 / BN;      // B rows per 1 KiB run (BN <= 256)
+  static constexpr int kRunB = 256 + 2048 / BN;      // floats between runs
+  static constexpr int kRunsB = BK * BN / 256;
+  static constexpr int kFloatsB = kRunsB * kRunB;
+  static constexpr int kStageFloats = kFloatsA + kFloatsB;
+  static constexpr int kStages = 3;
+  static constexpr int kLdsBytes = kStages * kStageFloats * 4;
+  static constexpr int kInstrA = kFloatsA / 256 / kWaves;  // 1 KiB loads per wave and slice
+  static constexpr int kInstrB = kRunsB / kWaves;
+  static constexpr int kSteps = BK / 2;
+  static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tile");
+  static_assert(BK == 16 || BK == 32, "K slice");
+  static_assert(BN == 64 || BN == 128 || BN == 256, "B rows per run");
+  static_assert(kFloatsA % (256 * kWaves) == 0 && kRunsB % kWaves == 0, "load split");
+  __host__ __device__ static constexpr int fa(int row) {
+    return ((row / kRp128A) % kCprA) ^ ((row / (kRp128A * kCprA)) & 1);
+  }
+  // float offset of B row k inside a stage's B region
+  __host__ __device__ static constexpr int brow(int k) {
+    return (k / kRowsPerRunB) * kRunB + (k % kRowsPerRunB) * BN;
+  }
+};
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, int MIN_WAVES>
+__global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_dl_kernel(
+    const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
+    int K, int tiles_m, int tiles_n, int group_m) {
+  using T = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>;
+  extern __shared__ __align__(16) float lds[];
+
+  const int logical = xcd_contiguous_id(blockIdx.x, tiles_m * tiles_n);
+  const int width = group_m * tiles_n;
+  const int group = logical / width;
+  const int first_m = group * group_m;
+  const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+  const int in_group = logical - group * width;
+  const int tile_m = first_m + in_group % gsz;
+  const int tile_n = in_group / gsz;
+  const int m0 = tile_m * BM;
+  const int n0 = tile_n * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N;
+  const int wn = wave % WAVES_N;
+  const int r32 = lane & 31;
+  const int half = lane >> 5;
+
+  float16_t acc[T::kTilesM][T::kTilesN];
+#pragma unroll
+  for (int i = 0; i < T::kTilesM; ++i)
+#pragma unroll
+    for (int j = 0; j < T::kTilesN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  // ---- direct loads: uniform slice base + per-lane 32-bit byte offsets ----
+  unsigned oa[T::kInstrA];
+  unsigned ob[T::kInstrB];
+#pragma unroll
+  for (int i = 0; i < T::kInstrA; ++i) {
+    const int idx = (wave * T::kInstrA + i) * 256 + lane * 4;  // float index in the LDS A tile
+    const int row = idx / BK;
+    const int c_log = ((idx % BK) / 4) ^ T::fa(row);
+    oa[i] = static_cast<unsigned>(row * K + 4 * c_log) * 4u;
+  }
+#pragma unroll
+  for (int i = 0; i < T::kInstrB; ++i) {
+    const int idx = (wave * T::kInstrB + i) * 256 + lane * 4;  // float index in the unpadded B tile
+    ob[i] = static_cast<unsigned>((idx / BN) * N + idx % BN) * 4u;
+  }
+  const char *ga = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
+  const char *gb = reinterpret_cast<const char *>(B + n0);
+  const int64_t b_step = static_cast<int64_t>(BK) * N * 4;
+  constexpr int kLoadsPerSlice = T::kInstrA + T::kInstrB;
+  // load l of the slice at (ga, gb) into the stage at float offset stage_off
+  auto issue_one = [&](int stage_off, int l) {
+    if (l < T::kInstrA) {
+      float *sa = lds + stage_off + (wave * T::kInstrA + l) * 256;
+      __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(ga + oa[l]), KCG_LDS_PTR(sa), 16, 0, 0);
+    } else {
+      const int i = l - T::kInstrA;
+      float *sb = lds + stage_off + T::kFloatsA + (wave * T::kInstrB + i) * T::kRunB;
+      __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(gb + ob[i]), KCG_LDS_PTR(sb), 16, 0, 0);
+    }
+  };
+  // The loop body is kept free of branches (after a join the compiler's wait-count
+  // tracking turns imprecise and drains the operand prefetch): past the last
+  // slice the pointers simply stop advancing and the final slice is fetched again
+  // into a stage nobody reads any more.
+  auto advance_if = [&](bool cond) {
+    ga += cond ? BK * 4 : 0;
+    gb += cond ? b_step : 0;
+  };
+
+  // ---- operand reads ----
+  // While a direct load is in flight the compiler treats the LDS counter as
+  // unordered and would wait for ALL outstanding LDS reads (lgkmcnt(0)) before
+  // every MFMA group, which undoes the operand prefetch.  The reads are therefore
+  // issued from inline assembly, invisible to that bookkeeping, and waited for by
+  // hand: LDS reads return in order, so "all but the newest n" is lgkmcnt(n).
+  int a_off[BK / 8];  // byte offsets inside a stage, swizzle folded in
+#pragma unroll
+  for (int kk = 0; kk < BK / 8; ++kk)
+    a_off[kk] = ((wm * T::kWaveM + r32) * BK + 4 * ((2 * kk) ^ half ^ T::fa(r32))) * 4;
+  const int b_off = (T::kFloatsA + half * T::brow(4) + wn * T::kWaveN + r32) * 4;
+
+  float4_t fa[2][T::kTilesM];
+  float fb[2][T::kTilesN];
+  float4_t na[T::kTilesM];
+  float nb[T::kTilesN];
+  // stage_addr: LDS byte address of the stage
+  auto read_a = [&](int stage_addr, int kk, float4_t(&dst)[T::kTilesM]) {
+    const int addr = stage_addr + a_off[kk];
+#pragma unroll
+    for (int i = 0; i < T::kTilesM; ++i)
+      asm volatile("ds_read_b128 %0, %1 offset:%2"
+                   : "=v"(dst[i])
+                   : "v"(addr), "n"(i * 32 * BK * 4)
+                   : "memory");
+  };
+  auto read_b = [&](int stage_addr, int s, float(&dst)[T::kTilesN]) {
+    const int addr = stage_addr + b_off;
+#pragma unroll
+    for (int n = 0; n < T::kTilesN; ++n)
+      asm volatile("ds_read_b32 %0, %1 offset:%2"
+                   : "=v"(dst[n])
+                   : "v"(addr), "n"((T::brow((s / 4) * 8 + s % 4) + n * 32) * 4)
+                   : "memory");
+  };
+  constexpr int kReadsA = T::kTilesM;  // LDS instructions per read_a / read_b
+  constexpr int kReadsB = T::kTilesN;
+  static_assert((T::brow(BK - 1) + BN) * 4 < 65536 && BM * BK * 4 < 65536, "ds_read offset field");
+  auto next_stage = [](int off) {
+    return off == (T::kStages - 1) * T::kStageFloats ? 0 : off + T::kStageFloats;
+  };
+  const int lds_base = static_cast<int>(reinterpret_cast<uintptr_t>(lds));
+
+  // Publishes the slice requested before the newest one: the wave waits for its
+  // own loads of that slice and for its LDS reads, then joins the barrier.  A bare
+  // s_barrier is used because __syncthreads() carries a release fence for which
+  // the compiler drains every outstanding load (vmcnt(0)), including the slice
+  // that was only just requested.
+  auto publish = [&]() {
+    // s_waitcnt vmcnt(kLoadsPerSlice) lgkmcnt(0), as the builtin so that the compiler's
+    // own wait-count bookkeeping sees it (encoding: vmcnt [3:0], expcnt [6:4], lgkmcnt [11:8])
+    static_assert(kLoadsPerSlice < 16, "vmcnt immediate");
+    __builtin_amdgcn_s_waitcnt(kLoadsPerSlice | 0x70);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  const int ktiles = K / BK;
+#pragma unroll
+  for (int l = 0; l < kLoadsPerSlice; ++l) issue_one(0, l);
+  advance_if(ktiles > 1);
+#pragma unroll
+  for (int l = 0; l < kLoadsPerSlice; ++l) issue_one(T::kStageFloats, l);
+  advance_if(ktiles > 2);
+  publish();
+  read_a(lds_base, 0, na);
+  read_b(lds_base, 0, nb);
+
+  int st = 0;  // stage (float offset) holding slice kt
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int st1 = next_stage(st);
+    const int st2 = next_stage(st1);
+    const int st_addr = lds_base + st * 4;
+    const int st1_addr = lds_base + st1 * 4;
+    // the reads of step 0, issued after the previous barrier, are the newest in flight
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < T::kTilesM; ++i) fa[0][i] = na[i];
+#pragma unroll
+    for (int n = 0; n < T::kTilesN; ++n) fb[0][n] = nb[n];
+#pragma unroll
+    for (int s = 0; s < T::kSteps; ++s) {
+      // The loads of slice kt+2 are spread over the steps: requests issued in one
+      // burst by every wave of the CU queue up at the address unit.
+#pragma unroll
+      for (int l = 0; l < kLoadsPerSlice; ++l)
+        if (s == 1 + l * (T::kSteps - 2) / kLoadsPerSlice) issue_one(st2, l);
+      if (s + 1 < T::kSteps) {
+        const bool with_a = (s + 1) % 4 == 0;
+        if (with_a) read_a(st_addr, (s + 1) / 4, fa[((s + 1) / 4) & 1]);
+        read_b(st_addr, s + 1, fb[(s + 1) & 1]);
+        // operands of step s were requested one step ago: all but this step's reads
+        if (with_a) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsA + kReadsB) : "memory");
+        else asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsB) : "memory");
+      } else {
+        publish();  // includes lgkmcnt(0): the operands of the last step are in
+        read_a(st1_addr, 0, na);
+        read_b(st1_addr, 0, nb);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < T::kTilesM; ++i)
+#pragma unroll
+        for (int n = 0; n < T::kTilesN; ++n)
+          acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[(s / 4) & 1][i][s % 4], fb[s & 1][n],
+                                                           acc[i][n], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    advance_if(kt + 3 < ktiles);
+    st = st1;
+  }
+  // LDS may be handed to another workgroup once this one retires: drain the loads.
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), lgkmcnt/expcnt untouched
+
+#pragma unroll
+  for (int i = 0; i < T::kTilesM; ++i) {
+#pragma unroll
+    for (int n = 0; n < T::kTilesN; ++n) {
+      const int col = n0 + wn * T::kWaveN + n * 32 + r32;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * T::kWaveM + i * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+        float v = acc[i][n][e];
+        if (RELU) v = relu_maxf(v);
+        C[static_cast<int64_t>(row) * N + col] = v;
       }
     }
   }
@@ -224,12 +531,33 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
     info->block[1] = info->block[2] = 1;
     info->lds_bytes = T::kLdsBytes;
     info->waves_per_block = WAVES_M * WAVES_N;
-    snprintf(info->kernel, sizeof info->kernel, "gemm_f32_%dx%dx%d_w%dx%d", BM, BN, BK, WAVES_M,
-             WAVES_N);
+    const char *kind = "";
+    if constexpr (BK == 16 || BK == 32) {
+      if (full) {  // the direct-load kernel takes full-tile problems
+        info->lds_bytes = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>::kLdsBytes;
+        kind = "_dl";
+      }
+    }
+    snprintf(info->kernel, sizeof info->kernel, "gemm_f32_%dx%dx%d_w%dx%d%s", BM, BN, BK, WAVES_M,
+             WAVES_N, kind);
     return KCG_OK;
   }
   dim3 grid(static_cast<unsigned>(tiles_m * tiles_n));
   dim3 block(T::kThreads);
+  if constexpr (BK == 16 || BK == 32) {
+    using TD = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>;
+    // the direct-load kernel addresses a slice with 32-bit byte offsets
+    if (full && K < (1 << 22) && N < (1 << 24)) {
+      auto launch_dl = [&](auto kern) {
+        if (!allow_lds(kern, TD::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
+        return launch(kern, grid, block, TD::kLdsBytes, stream, A, B, C, static_cast<int>(M),
+                      static_cast<int>(N), static_cast<int>(K), static_cast<int>(tiles_m),
+                      static_cast<int>(tiles_n), group_m);
+      };
+      return relu ? launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, true, MIN_WAVES>)
+                  : launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, MIN_WAVES>);
+    }
+  }
 #define KCG_LAUNCH(RELU_, FULL_)                                                                 \
   do {                                                                                           \
     auto kern = gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N, RELU_, FULL_, MIN_WAVES>;          \
@@ -299,7 +627,6 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
   KCG_TRY(128, 128, 8, 2, 2, 2)
   KCG_TRY(256, 128, 16, 4, 2, 2)
   KCG_TRY(256, 128, 32, 4, 2, 1)
-  KCG_TRY(256, 256, 16, 2, 2, 1)
   KCG_TRY(64, 64, 32, 2, 2, 2)
 #undef KCG_TRY
   return KCG_ERR_BAD_SCHEDULE;
