@@ -24,7 +24,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 # HBM bytes per launch (fetch + write) measured with rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE, each scaled by the same counter's reading for a 256 MiB copy
 # (profiles/gemm_f32_cfg1.md, profiles/fmha_f32_cfg3.md, profiles/fmha_bf16_cfg4.md).
-TRAFFIC_BYTES = {"gemm_cfg1": 916031389, "fmha_cfg3": 134384584, "fmha_cfg4": 795121940}
+TRAFFIC_BYTES = {"gemm_cfg1": 771442602, "fmha_cfg3": 134384584, "fmha_cfg4": 795121940}
 
 
 def time_launches(fn, steps, warmup):
@@ -100,7 +100,7 @@ def main():
         "pct_fp32_peak": round(100.0 * value / PEAK_FP32_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_TFLOPS, 4),
-                     "traffic": TRAFFIC_BYTES["gemm_cfg1"], "kernel": "gemm_f32_kernel",
+                     "traffic": TRAFFIC_BYTES["gemm_cfg1"], "kernel": "gemm_f32_dl_kernel",
                      "algorithmic_flops": flops, "algorithmic_bytes": alg_bytes,
                      "launch_ms": round(ev_ms, 5)},
     }
