@@ -65,6 +65,13 @@ class KernelCodeGenerator {
 
   void setLogMode(Log level) { KCGLog::level = level; }
 
+  // Replaces the two config tables by the gfx950 search space: every tile shape
+  // the kernel library builds.  Meant for use with a measured evaluator; with
+  // the default evaluate() (constant 0) the first entry still wins.
+  void useCandidateTables();
+  // evaluate() of the module optimize() returned (FLT_MAX before any call).
+  float bestLatency() const { return minLatency; }
+
   std::vector<std::map<std::string, int>> matmulConfigs;
   std::vector<std::map<std::string, int>> fmhaConfigs;
 

@@ -25,6 +25,24 @@ KernelCodeGenerator::KernelCodeGenerator(const std::string &platform_) : platfor
   };
 }
 
+void KernelCodeGenerator::useCandidateTables() {
+  auto mm = [](int bm, int bn, int bk, int wm, int wn) {
+    return std::map<std::string, int>{{"BLOCK_SIZE_M", bm}, {"BLOCK_SIZE_N", bn}, {"BLOCK_SIZE_K", bk},
+                                      {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 8}, {"THREAD_SIZE_N", 8},
+                                      {"WAVE_SIZE_M", wm}, {"WAVE_SIZE_N", wn}, {"VECTORIZE_WIDTH", 4},
+                                      {"WARP_SIZE", 64}};
+  };
+  matmulConfigs = {mm(256, 128, 16, 64, 64), mm(256, 128, 32, 64, 64), mm(128, 128, 16, 64, 64),
+                   mm(128, 128, 32, 64, 64), mm(128, 128, 8, 64, 64),  mm(64, 64, 32, 32, 32)};
+  // fp32 attention is built for Br 128 x Bc 32|64, bf16 for Br 128|256 x Bc 64; candidates a
+  // data type has no kernel for are refused at bind time and score FLT_MAX.
+  fmhaConfigs = {
+      {{"BLOCK_SIZE", 256}, {"Br", 128}, {"Bc", 32}, {"WARP_SIZE", 64}},
+      {{"BLOCK_SIZE", 256}, {"Br", 128}, {"Bc", 64}, {"WARP_SIZE", 64}},
+      {{"BLOCK_SIZE", 512}, {"Br", 256}, {"Bc", 64}, {"WARP_SIZE", 64}},
+  };
+}
+
 ComputeDAG &KernelCodeGenerator::createGraph(const std::string &graphName) {
   minLatency = FLT_MAX;
   graph.module = ir::ModuleOp::create(graphName);

@@ -3,6 +3,13 @@
 //
 //   demo_rocm matmul M N K relu(0|1) out.bin
 //   demo_rocm fmha   B H S D causal(0|1) scale out.bin
+//   demo_rocm tune matmul M N K relu(0|1) out.bin
+//   demo_rocm tune fmha   B H S D causal(0|1) scale out.bin
+//
+// The tune forms run the reference's config trial loop (src/KernelCodeGen.cc:15-51)
+// with a measured evaluate(): every candidate schedule is timed on the device,
+// the trials are printed as "trial <schedule> <kernel> <ms|refused>", the winner
+// as "best <schedule> <ms>", and the winner's output is written to out.bin.
 //
 // Builds the graph through KernelCodeGenerator, optimizes it, binds the result
 // to the gfx950 kernel, runs it on seeded uniform[-1,1) inputs (the generator of
@@ -16,6 +23,7 @@
 #include <string>
 #include <vector>
 
+#include "Backend/HIPTimer.h"
 #include "KernelCodeGen.h"
 
 using namespace KernelCodeGen;
@@ -75,11 +83,36 @@ static int run(const KernelBinding &b, const std::vector<std::vector<float> *> &
 
 int main(int argc, char **argv) {
   if (argc < 2) {
-    std::fprintf(stderr, "usage: demo_rocm matmul M N K relu out | demo_rocm fmha B H S D causal scale out\n");
+    std::fprintf(stderr, "usage: demo_rocm [tune] matmul M N K relu out | demo_rocm [tune] fmha B H S D causal scale out\n");
     return 1;
   }
   KernelCodeGenerator generator("ROCm");
   generator.setLogMode(Log::Release);
+  HIPTimer timer(3, 20);
+  bool tune = false;
+  if (std::string(argv[1]) == "tune") {
+    tune = true;
+    generator.useCandidateTables();
+    generator.setEvaluator([&](ir::ModuleOp &m) { return timer(m); });
+    --argc;
+    ++argv;
+  }
+  auto report = [&](const std::vector<KernelBinding> &bindings) {
+    if (!tune) return;
+    for (auto &t : timer.trials()) {
+      if (t.status == KCG_OK) std::printf("trial %s %s %.5f\n", t.schedule.c_str(), t.kernel.c_str(), t.ms);
+      else std::printf("trial %s - refused\n", t.schedule.c_str());
+    }
+    if (!bindings.empty()) {
+      const KernelBinding &b = bindings[0];
+      char sched[64];
+      if (b.kind == KernelBinding::Gemm)
+        std::snprintf(sched, sizeof sched, "%dx%dx%d", b.gemmSched.block_m, b.gemmSched.block_n, b.gemmSched.block_k);
+      else
+        std::snprintf(sched, sizeof sched, "br%d bc%d", b.fmhaSched.br, b.fmhaSched.bc);
+      std::printf("best %s %.5f\n", sched, generator.bestLatency());
+    }
+  };
   const std::string mode = argv[1];
   if (mode == "matmul" && argc == 7) {
     const int64_t m = std::atoll(argv[2]), n = std::atoll(argv[3]), k = std::atoll(argv[4]);
@@ -92,6 +125,7 @@ int main(int argc, char **argv) {
     auto module = generator.optimize(graph);
     auto bindings = generator.bind(module);
     if (bindings.size() != 1) return 5;
+    report(bindings);
     std::printf("%s", generator.codegen(module).c_str());
     std::vector<float> a(m * k), b(k * n);
     fill_uniform(a, kSeed, 0);
@@ -113,6 +147,7 @@ int main(int argc, char **argv) {
     auto module = generator.optimize(graph);
     auto bindings = generator.bind(module);
     if (bindings.size() != 1) return 5;
+    report(bindings);
     std::printf("%s", generator.codegen(module).c_str());
     const size_t count = static_cast<size_t>(bsz * h * s * d);
     std::vector<float> q(count), kk(count), v(count);

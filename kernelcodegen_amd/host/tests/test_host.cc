@@ -524,6 +524,28 @@ static void test_facade_config_search_and_reference_tile() {
   auto second = generator.bind(generator.optimize(graph));
   CHECK(second.size() == 1 && second[0].gemmSched.block_m == 128 && second[0].gemmSched.block_k == 8);
   CHECK(second[0].launch.grid[0] == 16 && second[0].launch.block[0] == 256);
+  // the gfx950 search space: every candidate is tried once, the cheapest one is kept,
+  // and a candidate the evaluator refuses (FLT_MAX) can never win
+  generator.useCandidateTables();
+  CHECK(generator.matmulConfigs.size() == 6 && generator.fmhaConfigs.size() == 3);
+  std::vector<std::string> seen;
+  generator.setEvaluator([&](ModuleOp &m) {
+    FuncOp f = Analyzer::collectFunctions(m, "Matmul_m")[0];
+    const std::string tile = f.getAttr("kcg.BLOCK_SIZE_M") + "x" + f.getAttr("kcg.BLOCK_SIZE_N") + "x" +
+                             f.getAttr("kcg.BLOCK_SIZE_K");
+    seen.push_back(tile);
+    if (tile == "64x64x32") return FLT_MAX;
+    return tile == "128x128x32" ? 0.5f : 1.0f + static_cast<float>(seen.size());
+  });
+  auto third = generator.bind(generator.optimize(graph));
+  CHECK(seen.size() == 6);
+  CHECK(third.size() == 1 && third[0].gemmSched.block_m == 128 && third[0].gemmSched.block_k == 32);
+  CHECK(generator.bestLatency() == 0.5f);
+  // nothing acceptable: the module stays un-scheduled and nothing binds
+  generator.setEvaluator([](ModuleOp &) { return FLT_MAX; });
+  std::vector<KernelBinding> none;
+  quiet([&] { none = generator.bind(generator.optimize(graph)); });
+  CHECK(none.empty());
 }
 
 // test/test.cc:64-107 of the reference: the attention graph through the facade.

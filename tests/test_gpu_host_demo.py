@@ -47,3 +47,48 @@ def test_flash_attention_demo(oracle, dev, tmp_path, causal):
     Q, K, V = (inputs.uniform((B, H, S, D), SEED, i) for i in range(3))
     ref = oracle.fmha(Q, K, V, scale=scale, causal=bool(causal), stable=True)
     assert max(rel_err(got.reshape(B, H, S, D), ref)) < 1e-4
+
+
+def _trials(text):
+    trials, best = [], None
+    for line in text.splitlines():
+        f = line.split()
+        if f and f[0] == "trial":
+            trials.append((" ".join(f[1:-2]), f[-2], None if f[-1] == "refused" else float(f[-1])))
+        elif f and f[0] == "best":
+            best = (" ".join(f[1:-1]), float(f[-1]))
+    return trials, best
+
+
+def test_matmul_config_search(oracle, dev, tmp_path):
+    """The trial loop with a measured evaluate(): every tile of the search space is timed on
+    the device, the fastest one is bound, and its result is still the oracle's."""
+    M, N, K = 2048, 2048, 1024
+    got, text = _run(["tune", "matmul", M, N, K, 1], tmp_path)
+    trials, best = _trials(text)
+    assert [t[0] for t in trials] == ["256x128x16", "256x128x32", "128x128x16", "128x128x32", "128x128x8", "64x64x32"]
+    timed = [t for t in trials if t[2] is not None]
+    assert len(timed) == 6 and all(0 < t[2] < 50 for t in timed)
+    fastest = min(timed, key=lambda t: t[2])
+    assert best is not None and best[0] == fastest[0] and abs(best[1] - fastest[2]) < 1e-4
+    bm, bn, bk = (int(x) for x in best[0].split("x"))
+    assert "static const kcg_gemm_sched sched = {%d, %d, %d," % (bm, bn, bk) in text
+    A = inputs.uniform((M, K), SEED, 0)
+    B = inputs.uniform((K, N), SEED, 1)
+    ref = oracle.relu(oracle.matmul(A, B))
+    assert max(rel_err(got.reshape(M, N), ref)) < 1e-4
+
+
+def test_attention_config_search(oracle, dev, tmp_path):
+    """fp32 attention: Br 128 x Bc 32|64 are timed, the 256-row block (bf16 only) is refused."""
+    B, H, S, D = 1, 8, 1024, 128
+    scale = D ** -0.5
+    got, text = _run(["tune", "fmha", B, H, S, D, 1, scale], tmp_path)
+    trials, best = _trials(text)
+    assert [t[0] for t in trials] == ["br128 bc32", "br128 bc64", "br256 bc64"]
+    assert trials[0][2] is not None and trials[1][2] is not None and trials[2][2] is None
+    fastest = min(trials[:2], key=lambda t: t[2])
+    assert best is not None and best[0] == fastest[0]
+    Q, K, V = (inputs.uniform((B, H, S, D), SEED, i) for i in range(3))
+    ref = oracle.fmha(Q, K, V, scale=scale, causal=True, stable=True)
+    assert max(rel_err(got.reshape(B, H, S, D), ref)) < 1e-4
