@@ -4,13 +4,17 @@
 // Frontend operators, the schedule primitives and the backend binding need:
 //
 //   module { memref.alloc ; func.func { affine.for / affine.parallel nests with
-//   affine.load / affine.store on linear index expressions, arith.{constant,
-//   mulf, addf, maxf, divf}, math.exp, affine.apply, affine.yield, gpu.barrier,
-//   func.return } ; func.call }
+//   affine.load / affine.store (scalar or affine.vector_load / vector_store of w
+//   contiguous elements) on linear index expressions, arith.{constant, mulf,
+//   addf, maxf, divf}, math.exp, affine.apply, affine.if, affine.yield,
+//   gpu.barrier, func.return } ; func.call }
 //
 // Index expressions are linear forms  sum(coeff_i * value_i) + constant  over
-// loop induction variables and affine.apply results, which is all that
-// split / reorder / parallel / bufferize ever create.
+// loop induction variables and affine.apply results.  floordiv / mod by a
+// constant (thread-id decompositions, double-buffer selectors) are affine.apply
+// ops of their own -- `(expr) floordiv c`, `(expr) mod c` -- whose results are
+// ordinary index values; the printer folds them back into the subscripts that
+// use them, so the text reads like MLIR's single-map form.
 //
 // Ownership: an Op owns its results, its block arguments (induction variables,
 // iter_args, function arguments) and the ops of its single-block region.
@@ -53,7 +57,8 @@ struct ValueImpl {
   int index = 0;
   bool isMemRef = false;
   MemRefType memref;
-  DType dtype = DType::none;  // scalar type when !isMemRef
+  DType dtype = DType::none;  // scalar (or vector element) type when !isMemRef
+  int lanes = 1;              // > 1: vector<lanes x dtype> (result of a vector load)
 };
 
 // Non-owning handle; null-testable like the reference's mlir::Value.
@@ -93,7 +98,7 @@ struct LinExpr {
 
 enum class OpKind {
   Module, Func, Alloc, Call, Return, For, Parallel, Apply, Load, Store, Constant,
-  MulF, AddF, MaxF, DivF, Exp, Yield, Barrier
+  MulF, AddF, MaxF, DivF, Exp, Yield, Barrier, If
 };
 
 const char *opName(OpKind k);  // "affine.for", ...
@@ -103,11 +108,12 @@ using OpList = std::list<std::unique_ptr<Op>>;
 struct Op {
   OpKind kind;
   Op *parent = nullptr;
-  OpList body;                    // Module / Func / For / Parallel
+  OpList body;                    // Module / Func / For / Parallel / If
   std::vector<Value> operands;    // arith operands; call / return / yield operands; store value;
                                   // for: iter_arg initial values
   Value memref;                   // load / store
-  std::vector<LinExpr> indices;   // load / store subscripts; apply: one expression
+  std::vector<LinExpr> indices;   // load / store subscripts; apply: one expression;
+                                  // if: constraints, each meaning expr >= 0
   std::vector<std::unique_ptr<ValueImpl>> results;
   std::vector<std::unique_ptr<ValueImpl>> args;  // for: iv [+ iter_args]; parallel: ivs; func: args
   int64_t lb = 0, ub = 0, step = 1;              // for
@@ -115,13 +121,18 @@ struct Op {
   std::string name;                              // module / func symbol, call callee
   std::map<std::string, std::string> attrs;      // e.g. func.state, affine.loop
   double fvalue = 0.0;                           // constant
+  int64_t divisor = 0;                           // apply: > 0 -> floordiv / mod by it
+  bool isMod = false;                            // apply: mod instead of floordiv
+  int vec = 0;                                   // load / store: 0 = scalar op, w >= 1 =
+                                                 // vector op on w contiguous elements
   std::vector<MemRefType> resultTypes;           // func signature results
 
   explicit Op(OpKind k) : kind(k) {}
   Value result(int i = 0) const { return Value(results[i].get()); }
   Value arg(int i) const { return Value(args[i].get()); }
   bool hasRegion() const {
-    return kind == OpKind::Module || kind == OpKind::Func || kind == OpKind::For || kind == OpKind::Parallel;
+    return kind == OpKind::Module || kind == OpKind::Func || kind == OpKind::For ||
+           kind == OpKind::Parallel || kind == OpKind::If;
   }
   // position helpers (this op inside parent->body)
   OpList::iterator self();
@@ -150,8 +161,15 @@ std::unique_ptr<Op> makeReturn(const std::vector<Value> &operands);
 std::unique_ptr<Op> makeFor(int64_t lb, int64_t ub, int64_t step, const std::vector<Value> &iterInits = {});
 std::unique_ptr<Op> makeParallel(const std::vector<int64_t> &ubs);
 std::unique_ptr<Op> makeApply(const LinExpr &e);
+std::unique_ptr<Op> makeApplyFloorDiv(const LinExpr &e, int64_t divisor);  // (e) floordiv divisor
+std::unique_ptr<Op> makeApplyMod(const LinExpr &e, int64_t divisor);       // (e) mod divisor
 std::unique_ptr<Op> makeLoad(Value memref, const std::vector<LinExpr> &idx);
 std::unique_ptr<Op> makeStore(Value value, Value memref, const std::vector<LinExpr> &idx);
+// width elements along the last dimension, starting at the subscript
+std::unique_ptr<Op> makeVectorLoad(Value memref, const std::vector<LinExpr> &idx, int width);
+std::unique_ptr<Op> makeVectorStore(Value value, Value memref, const std::vector<LinExpr> &idx, int width);
+// affine.if: the body runs when every constraint evaluates >= 0 (no else region)
+std::unique_ptr<Op> makeIf(const std::vector<LinExpr> &constraints);
 std::unique_ptr<Op> makeConstant(double v, DType t);
 std::unique_ptr<Op> makeBinary(OpKind k, Value a, Value b);
 std::unique_ptr<Op> makeExp(Value a);
@@ -194,6 +212,11 @@ struct ForOp : OpHandle {
   int64_t getStep() const { return op->step; }
   int64_t tripCount() const { return (op->ub - op->lb + op->step - 1) / op->step; }
   size_t numIterArgs() const { return op->args.size() - 1; }
+};
+
+struct IfOp : OpHandle {
+  using OpHandle::OpHandle;
+  const std::vector<LinExpr> &getConstraints() const { return op->indices; }
 };
 
 struct ParallelOp : OpHandle {

@@ -104,6 +104,7 @@ const char *opName(OpKind k) {
     case OpKind::Exp: return "math.exp";
     case OpKind::Yield: return "affine.yield";
     case OpKind::Barrier: return "gpu.barrier";
+    case OpKind::If: return "affine.if";
   }
   return "?";
 }
@@ -280,6 +281,38 @@ std::unique_ptr<Op> makeApply(const LinExpr &e) {
   return op;
 }
 
+std::unique_ptr<Op> makeApplyFloorDiv(const LinExpr &e, int64_t divisor) {
+  auto op = makeApply(e);
+  op->divisor = divisor;
+  return op;
+}
+
+std::unique_ptr<Op> makeApplyMod(const LinExpr &e, int64_t divisor) {
+  auto op = makeApply(e);
+  op->divisor = divisor;
+  op->isMod = true;
+  return op;
+}
+
+std::unique_ptr<Op> makeVectorLoad(Value memref, const std::vector<LinExpr> &idx, int width) {
+  auto op = makeLoad(memref, idx);
+  op->vec = width;
+  op->results[0]->lanes = width;
+  return op;
+}
+
+std::unique_ptr<Op> makeVectorStore(Value value, Value memref, const std::vector<LinExpr> &idx, int width) {
+  auto op = makeStore(value, memref, idx);
+  op->vec = width;
+  return op;
+}
+
+std::unique_ptr<Op> makeIf(const std::vector<LinExpr> &constraints) {
+  auto op = std::make_unique<Op>(OpKind::If);
+  op->indices = constraints;
+  return op;
+}
+
 std::unique_ptr<Op> makeLoad(Value memref, const std::vector<LinExpr> &idx) {
   auto op = std::make_unique<Op>(OpKind::Load);
   op->memref = memref;
@@ -370,6 +403,9 @@ static std::unique_ptr<Op> cloneRec(const Op *op, std::map<ValueImpl *, ValueImp
   c->name = op->name;
   c->attrs = op->attrs;
   c->fvalue = op->fvalue;
+  c->divisor = op->divisor;
+  c->isMod = op->isMod;
+  c->vec = op->vec;
   c->resultTypes = op->resultTypes;
   auto copyVals = [&](const std::vector<std::unique_ptr<ValueImpl>> &src,
                       std::vector<std::unique_ptr<ValueImpl>> &dst) {
@@ -423,14 +459,31 @@ struct Printer {
   void defArgs(const Op *op) {
     for (auto &a : op->args) names[a.get()] = "%arg" + std::to_string(nextArg++);
   }
+  // `(inner) floordiv c` / `(inner) mod c` for a value defined by such an apply, else its name
+  std::string atom(Value v, bool &compound) {
+    compound = false;
+    const Op *def = v.getDefiningOp();
+    if (def && def->kind == OpKind::Apply && def->divisor > 0) {
+      const LinExpr &in = def->indices[0];
+      const bool simple = in.terms.size() == 1 && in.terms[0].second == 1 && in.constant == 0;
+      bool innerCompound = false;
+      std::string inner = simple ? atom(in.terms[0].first, innerCompound) : expr(in);
+      if (!simple || innerCompound) inner = "(" + inner + ")";
+      compound = true;
+      return inner + (def->isMod ? " mod " : " floordiv ") + std::to_string(def->divisor);
+    }
+    return name(v);
+  }
   std::string expr(const LinExpr &e) {
     std::ostringstream s;
     bool first = true;
     for (auto &t : e.terms) {
       if (!first) s << " + ";
       first = false;
-      s << name(t.first);
-      if (t.second != 1) s << " * " << t.second;
+      bool compound = false;
+      const std::string a = atom(t.first, compound);
+      if (t.second != 1) s << (compound ? "(" + a + ")" : a) << " * " << t.second;
+      else s << a;
     }
     if (e.constant != 0 || first) {
       if (!first) s << " + ";
@@ -553,6 +606,7 @@ struct Printer {
       }
       case OpKind::Apply: {
         defResult(op);
+        if (op->divisor > 0) break;  // folded into the expressions that use it
         indent(d);
         // affine_map<(d0) -> (d0 * 128)>(%arg0)
         const LinExpr &e = op->indices[0];
@@ -572,13 +626,17 @@ struct Printer {
       case OpKind::Load:
         defResult(op);
         indent(d);
-        os << name(op->result()) << " = affine.load " << name(op->memref) << subscripts(op) << " : "
-           << op->memref.getMemRefType().str() << "\n";
+        os << name(op->result()) << (op->vec ? " = affine.vector_load " : " = affine.load ") << name(op->memref)
+           << subscripts(op) << " : " << op->memref.getMemRefType().str();
+        if (op->vec) os << ", vector<" << op->vec << "x" << dtypeName(op->memref.getMemRefType().elem) << ">";
+        os << "\n";
         break;
       case OpKind::Store:
         indent(d);
-        os << "affine.store " << name(op->operands[0]) << ", " << name(op->memref) << subscripts(op)
-           << " : " << op->memref.getMemRefType().str() << "\n";
+        os << (op->vec ? "affine.vector_store " : "affine.store ") << name(op->operands[0]) << ", "
+           << name(op->memref) << subscripts(op) << " : " << op->memref.getMemRefType().str();
+        if (op->vec) os << ", vector<" << op->vec << "x" << dtypeName(op->memref.getMemRefType().elem) << ">";
+        os << "\n";
         break;
       case OpKind::Constant: {
         defResult(op);
@@ -615,7 +673,47 @@ struct Printer {
         indent(d);
         os << "gpu.barrier\n";
         break;
+      case OpKind::If: {
+        // affine.if affine_set<(d0) : (-d0 + 1008 >= 0)>(%arg4) {
+        std::vector<Value> dims;
+        for (auto &e : op->indices)
+          for (auto &t : e.terms) {
+            bool seen = false;
+            for (auto &v : dims) seen = seen || v == t.first;
+            if (!seen) dims.push_back(t.first);
+          }
+        indent(d);
+        os << "affine.if affine_set<(";
+        for (size_t i = 0; i < dims.size(); ++i) os << (i ? ", " : "") << "d" << i;
+        os << ") : (";
+        for (size_t c = 0; c < op->indices.size(); ++c) {
+          const LinExpr &e = op->indices[c];
+          if (c) os << ", ";
+          bool first = true;
+          for (auto &t : e.terms) {
+            size_t di = 0;
+            while (!(dims[di] == t.first)) ++di;
+            if (t.second == -1) os << (first ? "-" : " - ") << "d" << di;
+            else if (t.second == 1) os << (first ? "" : " + ") << "d" << di;
+            else os << (first ? "" : " + ") << "d" << di << " * " << t.second;
+            first = false;
+          }
+          if (e.constant != 0 || first) os << (first ? "" : " + ") << e.constant;
+          os << " >= 0";
+        }
+        os << ")>(";
+        for (size_t i = 0; i < dims.size(); ++i) os << (i ? ", " : "") << atomName(dims[i]);
+        os << ") {\n";
+        region(op, d + 1);
+        indent(d);
+        os << "}\n";
+        break;
+      }
     }
+  }
+  std::string atomName(Value v) {
+    bool c = false;
+    return atom(v, c);
   }
 };
 }  // namespace
@@ -655,6 +753,10 @@ struct Verifier {
         use(op, t.first);
         if (t.first && t.first.getDType() != DType::index) fail(op, "non-index value in an index expression");
       }
+    if (op->kind == OpKind::Apply && op->divisor < 0) fail(op, "negative divisor");
+    if ((op->kind == OpKind::Load || op->kind == OpKind::Store) && op->vec < 0) fail(op, "negative vector width");
+    if (op->kind == OpKind::Store && op->vec > 0 && op->operands[0] && op->operands[0].get()->lanes != op->vec)
+      fail(op, "vector store of a value with another width");
     if (op->kind == OpKind::For) {
       if (op->step <= 0) fail(op, "non-positive step");
       if (op->ub < op->lb) fail(op, "upper bound below lower bound");

@@ -17,25 +17,63 @@ float *Interpreter::alloc(const MemRefType &t) {
   return owned_.back().get();
 }
 
+float *Interpreter::getMem(Frame &fr, Value v) {
+  for (Frame *f = &fr; f; f = f->parent) {
+    auto it = f->mem.find(v.get());
+    if (it != f->mem.end()) return it->second;
+  }
+  return nullptr;
+}
+
+float Interpreter::getF(Frame &fr, Value v) {
+  for (Frame *f = &fr; f; f = f->parent) {
+    auto it = f->f.find(v.get());
+    if (it != f->f.end()) return it->second;
+  }
+  error_ = "scalar value used before definition";
+  return 0.0f;
+}
+
+const std::vector<float> *Interpreter::getV(Frame &fr, Value v) {
+  for (Frame *f = &fr; f; f = f->parent) {
+    auto it = f->v.find(v.get());
+    if (it != f->v.end()) return &it->second;
+  }
+  return nullptr;
+}
+
+bool Interpreter::getI(Frame &fr, Value v, int64_t &out) {
+  for (Frame *f = &fr; f; f = f->parent) {
+    auto it = f->i.find(v.get());
+    if (it != f->i.end()) {
+      out = it->second;
+      return true;
+    }
+  }
+  return false;
+}
+
 int64_t Interpreter::eval(const LinExpr &e, Frame &fr) {
   int64_t v = e.constant;
   for (auto &t : e.terms) {
-    auto it = fr.i.find(t.first.get());
-    if (it == fr.i.end()) {
+    int64_t x = 0;
+    if (!getI(fr, t.first, x)) {
       error_ = "index value used before definition";
       return 0;
     }
-    v += it->second * t.second;
+    v += x * t.second;
   }
   return v;
 }
 
 int64_t Interpreter::offset(const Op *op, Frame &fr) {
   const auto &shape = op->memref.getMemRefType().shape;
+  const int width = op->vec > 0 ? op->vec : 1;
   int64_t off = 0;
   for (size_t d = 0; d < shape.size(); ++d) {
     const int64_t idx = eval(op->indices[d], fr);
-    if (idx < 0 || idx >= shape[d]) {
+    const int64_t span = d + 1 == shape.size() ? width : 1;
+    if (idx < 0 || idx + span > shape[d]) {
       error_ = "subscript out of bounds";
       return 0;
     }
@@ -44,10 +82,68 @@ int64_t Interpreter::offset(const Op *op, Frame &fr) {
   return off;
 }
 
+bool Interpreter::holds(const Op *ifOp, Frame &fr) {
+  for (auto &c : ifOp->indices)
+    if (eval(c, fr) < 0) return false;
+  return true;
+}
+
+bool Interpreter::containsBarrier(const Op *op) {
+  auto it = barrierInside_.find(op);
+  if (it != barrierInside_.end()) return it->second;
+  bool any = op->kind == OpKind::Barrier;
+  for (auto &k : op->body) any = containsBarrier(k.get()) || any;
+  barrierInside_[op] = any;
+  return any;
+}
+
 void Interpreter::execRegion(const Op *op, Frame &fr) {
   for (auto &k : op->body) {
     if (!error_.empty()) return;
     exec(k.get(), fr);
+  }
+}
+
+void Interpreter::execLockStep(const OpList &body, std::vector<Frame> &threads) {
+  for (auto &kp : body) {
+    if (!error_.empty()) return;
+    const Op *k = kp.get();
+    if (!containsBarrier(k)) {
+      for (auto &t : threads) {
+        exec(k, t);
+        if (!error_.empty()) return;
+      }
+      continue;
+    }
+    switch (k->kind) {
+      case OpKind::Barrier:
+        break;  // every thread has finished the statements before it
+      case OpKind::For: {
+        const size_t nIter = k->args.size() - 1;
+        for (auto &t : threads)
+          for (size_t a = 0; a < nIter; ++a) t.f[k->args[a + 1].get()] = getF(t, k->operands[a]);
+        for (int64_t iv = k->lb; iv < k->ub && error_.empty(); iv += k->step) {
+          for (auto &t : threads) t.i[k->args[0].get()] = iv;
+          execLockStep(k->body, threads);
+          const Op *yield = k->body.back().get();
+          for (auto &t : threads)
+            for (size_t a = 0; a < nIter; ++a) t.f[k->args[a + 1].get()] = getF(t, yield->operands[a]);
+        }
+        for (auto &t : threads)
+          for (size_t a = 0; a < nIter; ++a) t.f[k->results[a].get()] = getF(t, k->args[a + 1].get());
+        break;
+      }
+      case OpKind::If: {
+        size_t yes = 0;
+        for (auto &t : threads) yes += holds(k, t) ? 1 : 0;
+        if (yes == threads.size()) execLockStep(k->body, threads);
+        else if (yes != 0) error_ = "gpu.barrier under a condition the threads of a block disagree on";
+        break;
+      }
+      default:
+        error_ = std::string("gpu.barrier inside ") + opName(k->kind) + " is not interpretable";
+        break;
+    }
   }
 }
 
@@ -59,78 +155,113 @@ void Interpreter::exec(const Op *op, Frame &fr) {
     case OpKind::Constant:
       fr.f[op->results[0].get()] = static_cast<float>(op->fvalue);
       break;
-    case OpKind::Apply:
-      fr.i[op->results[0].get()] = eval(op->indices[0], fr);
+    case OpKind::Apply: {
+      int64_t v = eval(op->indices[0], fr);
+      if (op->divisor > 0) {
+        int64_t q = v / op->divisor, r = v % op->divisor;
+        if (r < 0) {  // floor semantics
+          r += op->divisor;
+          q -= 1;
+        }
+        v = op->isMod ? r : q;
+      }
+      fr.i[op->results[0].get()] = v;
       break;
+    }
     case OpKind::Load: {
-      float *base = fr.mem[op->memref.get()];
+      float *base = getMem(fr, op->memref);
       if (!base) {
         error_ = "load from an unbound memref";
         return;
       }
       const int64_t off = offset(op, fr);
-      if (error_.empty()) fr.f[op->results[0].get()] = base[off];
+      if (!error_.empty()) return;
+      if (op->vec > 0) fr.v[op->results[0].get()] = std::vector<float>(base + off, base + off + op->vec);
+      else fr.f[op->results[0].get()] = base[off];
       break;
     }
     case OpKind::Store: {
-      float *base = fr.mem[op->memref.get()];
+      float *base = getMem(fr, op->memref);
       if (!base) {
         error_ = "store to an unbound memref";
         return;
       }
       const int64_t off = offset(op, fr);
-      if (error_.empty()) base[off] = fr.f[op->operands[0].get()];
+      if (!error_.empty()) return;
+      if (op->vec > 0) {
+        const std::vector<float> *v = getV(fr, op->operands[0]);
+        if (!v || static_cast<int>(v->size()) != op->vec) {
+          error_ = "vector store of a value that is not a vector of that width";
+          return;
+        }
+        for (int l = 0; l < op->vec; ++l) base[off + l] = (*v)[l];
+      } else {
+        base[off] = getF(fr, op->operands[0]);
+      }
       break;
     }
     case OpKind::MulF: {
-      volatile float r = fr.f[op->operands[0].get()] * fr.f[op->operands[1].get()];
+      volatile float r = getF(fr, op->operands[0]) * getF(fr, op->operands[1]);
       fr.f[op->results[0].get()] = r;
       break;
     }
     case OpKind::AddF: {
-      volatile float r = fr.f[op->operands[0].get()] + fr.f[op->operands[1].get()];
+      volatile float r = getF(fr, op->operands[0]) + getF(fr, op->operands[1]);
       fr.f[op->results[0].get()] = r;
       break;
     }
     case OpKind::DivF:
-      fr.f[op->results[0].get()] = fr.f[op->operands[0].get()] / fr.f[op->operands[1].get()];
+      fr.f[op->results[0].get()] = getF(fr, op->operands[0]) / getF(fr, op->operands[1]);
       break;
     case OpKind::MaxF: {
-      const float a = fr.f[op->operands[0].get()], b = fr.f[op->operands[1].get()];
+      const float a = getF(fr, op->operands[0]), b = getF(fr, op->operands[1]);
       fr.f[op->results[0].get()] = (a != a) ? a : (b != b) ? b : (a > b ? a : b);
       break;
     }
     case OpKind::Exp:
-      fr.f[op->results[0].get()] = std::exp(fr.f[op->operands[0].get()]);
+      fr.f[op->results[0].get()] = std::exp(getF(fr, op->operands[0]));
       break;
     case OpKind::For: {
       const size_t nIter = op->args.size() - 1;
-      for (size_t a = 0; a < nIter; ++a) fr.f[op->args[a + 1].get()] = fr.f[op->operands[a].get()];
+      for (size_t a = 0; a < nIter; ++a) fr.f[op->args[a + 1].get()] = getF(fr, op->operands[a]);
       for (int64_t iv = op->lb; iv < op->ub && error_.empty(); iv += op->step) {
         fr.i[op->args[0].get()] = iv;
         execRegion(op, fr);
         const Op *yield = op->body.back().get();
-        for (size_t a = 0; a < nIter; ++a) fr.f[op->args[a + 1].get()] = fr.f[yield->operands[a].get()];
+        for (size_t a = 0; a < nIter; ++a) fr.f[op->args[a + 1].get()] = getF(fr, yield->operands[a]);
       }
-      for (size_t a = 0; a < nIter; ++a) fr.f[op->results[a].get()] = fr.f[op->args[a + 1].get()];
+      for (size_t a = 0; a < nIter; ++a) fr.f[op->results[a].get()] = getF(fr, op->args[a + 1].get());
       break;
     }
+    case OpKind::If:
+      if (holds(op, fr)) execRegion(op, fr);
+      break;
     case OpKind::Parallel: {
-      std::vector<int64_t> idx(op->ubs.size(), 0);
       int64_t total = 1;
       for (auto u : op->ubs) total *= u;
-      ++parallelDepth_;
-      for (int64_t n = 0; n < total && error_.empty(); ++n) {
-        int64_t r = n;
+      auto setIvs = [&](Frame &f, int64_t n) {
         for (int d = static_cast<int>(op->ubs.size()) - 1; d >= 0; --d) {
-          fr.i[op->args[d].get()] = r % op->ubs[d];
-          r /= op->ubs[d];
+          f.i[op->args[d].get()] = n % op->ubs[d];
+          n /= op->ubs[d];
         }
-        // a buffer allocated inside the body is private to one index point; index
-        // points run one after the other here, so its storage is simply reused
-        execRegion(op, fr);
+      };
+      if (containsBarrier(op)) {
+        // a thread block: one frame per index point, walked in lock step
+        std::vector<Frame> threads(static_cast<size_t>(total));
+        for (int64_t n = 0; n < total; ++n) {
+          threads[n].parent = &fr;
+          setIvs(threads[n], n);
+        }
+        execLockStep(op->body, threads);
+      } else {
+        for (int64_t n = 0; n < total && error_.empty(); ++n) {
+          // a buffer allocated inside the body is private to one index point
+          Frame point;
+          point.parent = &fr;
+          setIvs(point, n);
+          execRegion(op, point);
+        }
       }
-      --parallelDepth_;
       break;
     }
     case OpKind::Call: {
@@ -143,7 +274,7 @@ void Interpreter::exec(const Op *op, Frame &fr) {
       }
       Frame inner;
       for (size_t a = 0; a < callee->args.size(); ++a) {
-        float *p = fr.mem[op->operands[a].get()];
+        float *p = getMem(fr, op->operands[a]);
         if (!p) {
           // an output buffer that nothing bound: allocate it on first use
           p = alloc(op->operands[a].getMemRefType());
@@ -154,12 +285,10 @@ void Interpreter::exec(const Op *op, Frame &fr) {
       execRegion(callee, inner);
       const Op *ret = callee->body.back().get();
       for (size_t r = 0; r < op->results.size() && r < ret->operands.size(); ++r)
-        fr.mem[op->results[r].get()] = inner.mem[ret->operands[r].get()];
+        fr.mem[op->results[r].get()] = getMem(inner, ret->operands[r]);
       break;
     }
-    case OpKind::Barrier:
-      if (parallelDepth_ > 0) error_ = "gpu.barrier inside affine.parallel is not interpretable";
-      break;
+    case OpKind::Barrier:  // outside any parallel level there is one thread: nothing to wait for
     case OpKind::Yield:
     case OpKind::Return:
     case OpKind::Func:
