@@ -14,6 +14,7 @@
 #include "Frontend/Operators.h"
 #include "IR/IR.h"
 #include "Optimizer/Analyzer.h"
+#include "IR/AffineMap.h"
 #include "Optimizer/Rewriter.h"
 
 // What a BatchMatmul_<batch..>_m<M>_n<N>_k<K>_<N|T><N|T> function name encodes.
@@ -46,6 +47,19 @@ struct Optimizer {
 // tile, k hoisted over (mi, ni) and split by BLOCK_SIZE_K.  A Relu applied in
 // place to the matmul's only result is folded into the kernel's epilogue
 // (extension; the reference leaves Relu un-generated).
+//
+// Config key SCHEDULE_DETAIL selects how far the recipe of the reference
+// (src/Optimizer/Optimizer.cc:383-548) is carried on the IR:
+//   0 (default)  the tiling above; the backend only needs the tile sizes
+//   1            + staging: global -> registers -> shared tiles (read / write /
+//                barrier), shared -> register fragments, cache_read of A and B,
+//                vectorised write-back of the register tile (cache_write, vectorize)
+//   2            + double buffering of the shared tiles and of the fragments
+//                (pipeline), peeled last k step (detach_last_loop), the
+//                reference's statement order (schedule / extract_loop /
+//                change_double_buffer), affine.if clean-up and unrolling
+// Levels 1 and 2 follow the reference's thread organisation (8 x 8 register tile,
+// BLOCK_SIZE = 16 x THREAD_SIZE in both directions); other tile shapes stay at level 0.
 struct MatmulOptimizer : Optimizer {
   MatmulOptimizer() { name = "Matmul"; }
   bool applicable(ir::ModuleOp &module) override;
@@ -64,6 +78,10 @@ struct MatmulOptimizer : Optimizer {
   std::map<ir::FuncOp, MemoryBuffer, CompareFunc> matmulBuffers;
 
   static std::map<std::string, int> matmulConfig;
+  // Index maps of the staged schedule by name: loadTileA, loadTileB, storeTileA,
+  // storeTileB, loadFragA, loadFragB, cacheReadA, cacheReadB, cacheWriteC
+  // (the reference's getAffineMap, Optimizer.cc:272-380, for the current config).
+  static ir::AffineMap getAffineMap(const std::string &mapIdentifier);
 };
 
 // BatchedMatmul(Q, K^T) -> Softmax -> BatchedMatmul(P, V), each result used

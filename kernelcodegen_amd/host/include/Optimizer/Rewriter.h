@@ -1,8 +1,11 @@
 // Schedule primitives over the affine IR (reference: include/Optimizer/Rewriter.h).
 //
-// The four primitives the matmul and attention recipes are built from --
-// split, reorder, parallel, bufferizeLoopCarryVar -- plus buffer allocation,
-// barriers and the small builders the recipes use.  Every primitive keeps the
+// split, reorder, parallel and bufferizeLoopCarryVar tile the nest; read, write,
+// barrier, cache_read, cache_write and vectorize stage tiles through shared
+// memory and registers; pipeline, change_double_buffer, detach_last_loop,
+// schedule and extract_loop double-buffer and software-pipeline the staging;
+// take_off_true_if, delete_false_if, unroll and unrollAttribute clean up.  Plus
+// buffer allocation and the small builders the recipes use.  Every primitive keeps the
 // handles the caller already holds valid (a loop that is re-nested or loses its
 // iter_arg stays the same op), and reports a violated precondition by printing
 // a message and leaving the IR untouched instead of asserting.
@@ -10,6 +13,9 @@
 
 #include <vector>
 
+#include <functional>
+
+#include "IR/AffineMap.h"
 #include "IR/IR.h"
 #include "Optimizer/Analyzer.h"
 #include "enum.h"
@@ -72,6 +78,81 @@ struct Rewriter {
 
   // Marks loops with at most `maxTrips` iterations {affine.loop = "unroll"}.
   static void unrollAttribute(ir::ModuleOp module, int64_t maxTrips);
+  // Same with the reference's predicate form (src/Optimizer/Rewriter.cc:1574-1603).
+  static void unrollAttribute(ir::ModuleOp module, const std::function<bool(ir::ForOp)> &unrollCheckFn);
+
+  // ---- staging through registers and shared memory (Rewriter.cc:601-807 there) ----
+
+  // Copy loop  for i = 0 to dst.size / width:  dst[i * width .. +width) = src[map(operands, i)] .. +width)
+  // placed before / after `compute_at` or at the begin / end of its body.  `dst` is a
+  // one-dimensional register buffer; the loop's induction variable is bound to the
+  // map's dimension operands.size().  Returns the loop.
+  static ir::ForOp read(ir::Value src, ir::Value dst, const ir::AffineMap &map, std::vector<ir::Value> operands,
+                        int64_t width, ir::ForOp compute_at, Position pos);
+  // The same loop appended to `where`.
+  static ir::ForOp read(ir::OpHandle where, ir::Value src, ir::Value dst, const ir::AffineMap &map,
+                        std::vector<ir::Value> operands, int64_t width);
+
+  // Copy loop out of a one-dimensional register buffer `src`:
+  //   for i = 0 to src.size / width:  dst[map(operands, i)] .. +width) = src[i * width .. +width)
+  // When the map has two dimensions more than there are operands the vector is
+  // scattered element by element (an inner loop j < width binds the last
+  // dimension, src[i * width + j] goes to dst[map(operands, i, j)]): a transposing store.
+  static ir::ForOp write(ir::Value src, ir::Value dst, const ir::AffineMap &map, std::vector<ir::Value> operands,
+                         int64_t width, ir::ForOp compute_at, Position pos);
+  static ir::ForOp write(ir::OpHandle where, ir::Value src, ir::Value dst, const ir::AffineMap &map,
+                         std::vector<ir::Value> operands, int64_t width);
+
+  // Every scalar load of `src` inside `scope` becomes a load of cached[map(operands)].
+  static void cache_read(ir::ForOp scope, ir::Value src, ir::Value cached, const ir::AffineMap &map,
+                         const std::vector<ir::Value> &operands);
+  // Every scalar store to `src` inside `scope` is re-subscripted: src[map(operands)].
+  // (`cached` names the buffer the stored values come from; like the reference,
+  // Rewriter.cc:755-762, the store keeps its target.)
+  static void cache_write(ir::ForOp scope, ir::Value src, ir::Value cached, const ir::AffineMap &map,
+                          const std::vector<ir::Value> &operands);
+
+  // For every store to `dst` under `parallelLevel`: the loops that enclose it, outermost first.
+  static std::vector<std::vector<ir::ForOp>> get_write(ir::ParallelOp parallelLevel, ir::Value dst);
+
+  // Sets the step of `readOrWrite` (lower bound 0, step 1, trip count a multiple of
+  // `width`) to `width` and turns the loads and stores in its body into vector
+  // operations of that width.  Returns the loop (null on a violated precondition).
+  static ir::ForOp vectorize(ir::ForOp readOrWrite, int64_t width);
+
+  // ---- double buffering and software pipelining (Rewriter.cc:809-1284, 1614-1643) ----
+
+  // Double-buffers `buffer`, which the loops `readBodys` (inside `compute_at`, in
+  // program order) fill once per iteration of `compute_at`:
+  //   * the buffer gets a leading dimension of extent 2 (`buffer` is updated);
+  //   * copies of readBodys with iv = lower bound, filling half 0, are placed before compute_at;
+  //   * inside compute_at the original readBodys are moved into
+  //       affine.if (iv + 2 * step <= ub) { ... }
+  //     at the top of the body, fetch for iv + step and fill half (iv / step + 1) mod 2;
+  //   * every other access to the buffer reads half (iv / step) mod 2.
+  // Returns {prologue loops, in-loop loops}.
+  static std::vector<std::vector<ir::ForOp>> pipeline(std::vector<ir::ForOp> readBodys, ir::Value &buffer,
+                                                      ir::ForOp compute_at);
+  // Accesses to the double buffer `buffer` inside `forOp` switch to the other half.
+  static void change_double_buffer(ir::ForOp forOp, ir::Value buffer);
+  // Peels the last iteration: the loop stops one step early and a copy of its
+  // body with iv = ub - step follows it.
+  static void detach_last_loop(ir::ForOp forOp);
+  // Moves `srcOp` before / after `dstOp`, or to the end of the loop `dstOp`.
+  static void schedule(ir::Op *srcOp, ir::Op *dstOp, Position pos);
+  // Copy of `srcOp` with forOp's induction variable fixed to its value in
+  // iteration `iteration`, placed before `forOp`.  Returns the copy.
+  static ir::Op *extract_loop(ir::Op *srcOp, ir::ForOp forOp, int64_t iteration);
+
+  // ---- clean-up (Rewriter.cc:1359-1603) ----
+
+  // affine.if whose constraints hold for every value its operands can take
+  // (loop and parallel index ranges): the body is spliced in its place.
+  static void take_off_true_if(ir::ModuleOp module);
+  // affine.if with a constraint that holds for no value of its operands: removed.
+  static void delete_false_if(ir::ModuleOp module);
+  // Fully unrolls every loop for which `unrollCheckFn` returns true (innermost first).
+  static void unroll(ir::ModuleOp module, const std::function<bool(ir::ForOp)> &unrollCheckFn);
 };
 
 }  // namespace KernelCodeGen

@@ -91,8 +91,10 @@ bool Interpreter::holds(const Op *ifOp, Frame &fr) {
 bool Interpreter::containsBarrier(const Op *op) {
   auto it = barrierInside_.find(op);
   if (it != barrierInside_.end()) return it->second;
+  // a barrier belongs to the innermost parallel level around it
   bool any = op->kind == OpKind::Barrier;
-  for (auto &k : op->body) any = containsBarrier(k.get()) || any;
+  for (auto &k : op->body)
+    if (k->kind != OpKind::Parallel) any = containsBarrier(k.get()) || any;
   barrierInside_[op] = any;
   return any;
 }

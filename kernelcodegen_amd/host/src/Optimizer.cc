@@ -1,5 +1,7 @@
 #include "Optimizer/Optimizer.h"
 
+#include <algorithm>
+
 #include <cstdio>
 #include <iostream>
 
@@ -79,6 +81,102 @@ bool MatmulOptimizer::applicable(ModuleOp &module) {
   return !matmuls.empty();
 }
 
+namespace {
+
+// thread organisation of the staged schedule: warps as 2 x (warps / 2), the lanes
+// of a warp as 8 x (warp / 8), as in the reference for 8 warps of 32 lanes
+struct ThreadOrg {
+  int64_t bm, bn, bk, width, warp, blockDimY, blockDimX, warps, warpOrg[2], threadOrg[2];
+  int64_t fragA, fragB, ldgA, ldgB;
+  bool consistent;
+};
+
+ThreadOrg threadOrg(const std::map<std::string, int> &config) {
+  auto cfg = [&](const char *key, int fallback) {
+    auto it = config.find(key);
+    return static_cast<int64_t>(it == config.end() ? fallback : it->second);
+  };
+  ThreadOrg o{};
+  o.bm = cfg("BLOCK_SIZE_M", 128);
+  o.bn = cfg("BLOCK_SIZE_N", 128);
+  o.bk = cfg("BLOCK_SIZE_K", 8);
+  o.width = cfg("VECTORIZE_WIDTH", 4);
+  o.warp = cfg("WARP_SIZE", 64);
+  const int64_t tm = cfg("THREAD_SIZE_M", 8), tn = cfg("THREAD_SIZE_N", 8);
+  o.blockDimY = o.bm / tm;
+  o.blockDimX = o.bn / tn;
+  const int64_t threads = o.blockDimY * o.blockDimX;
+  o.warps = o.warp > 0 ? threads / o.warp : 0;
+  o.warpOrg[0] = 2;
+  o.warpOrg[1] = o.warps / 2;
+  o.threadOrg[0] = 8;
+  o.threadOrg[1] = o.warp / 8;
+  const int64_t strideA = o.warpOrg[1] > 0 ? (o.warps / o.warpOrg[1]) * o.threadOrg[0] : 0;
+  const int64_t strideB = (o.warps / o.warpOrg[0]) * o.threadOrg[1];
+  o.fragA = strideA > 0 ? o.bm / strideA : 0;
+  o.fragB = strideB > 0 ? o.bn / strideB : 0;
+  o.ldgA = threads > 0 ? o.bk * o.bm / threads : 0;
+  o.ldgB = threads > 0 ? o.bk * o.bn / threads : 0;
+  o.consistent = o.warps >= 2 && o.warps % 2 == 0 && o.warp % 8 == 0 && threads % o.warp == 0 &&
+                 o.fragA == tm && o.fragB == tn && o.width > 0 && o.fragA % o.width == 0 &&
+                 o.fragB % o.width == 0 && o.ldgA >= o.width && o.ldgA % o.width == 0 && o.ldgB >= o.width &&
+                 o.ldgB % o.width == 0 && o.bk % o.width == 0 && o.bn % o.width == 0 &&
+                 (o.bk * o.bm) % threads == 0 && (o.bk * o.bn) % threads == 0;
+  return o;
+}
+
+}  // namespace
+
+AffineMap MatmulOptimizer::getAffineMap(const std::string &id) {
+  const ThreadOrg o = threadOrg(matmulConfig);
+  auto d = [](int i) { return AffineExpr::dim(i); };
+  const int64_t w = o.width;
+  const AffineExpr tid = d(0) * o.blockDimX + d(1);
+  const AffineExpr warpId = tid.floorDiv(o.warp), laneId = tid % o.warp;
+  const int64_t threads = o.blockDimY * o.blockDimX;
+  if (id == "loadTileA") {
+    // operands: threadIdx.y, threadIdx.x, blockIdx.y, k_outer, copy step
+    const AffineExpr vt = tid + d(4) * threads;
+    return {5, {vt.floorDiv(o.bk / w) + d(2) * o.bm, (vt % (o.bk / w)) * w + d(3)}};
+  }
+  if (id == "loadTileB") {
+    // operands: threadIdx.y, threadIdx.x, k_outer, blockIdx.x, copy step
+    const AffineExpr vt = tid + d(4) * threads;
+    return {5, {vt.floorDiv(o.bn / w) + d(2), (vt % (o.bn / w)) * w + d(3) * o.bn}};
+  }
+  if (id == "storeTileA") {
+    // operands: threadIdx.y, threadIdx.x, copy step, element of the vector (transposing store)
+    const AffineExpr vt = tid + d(2) * threads;
+    return {4, {(vt % (o.bk / w)) * w + d(3), vt.floorDiv(o.bk / w)}};
+  }
+  if (id == "storeTileB") {
+    // operands: threadIdx.y, threadIdx.x, copy step
+    const AffineExpr vt = tid + d(2) * threads;
+    return {3, {vt.floorDiv(o.bn / w), (vt % (o.bn / w)) * w}};
+  }
+  if (id == "loadFragA") {
+    // operands: threadIdx.y, threadIdx.x, k_inner, copy step
+    const AffineExpr m = laneId.floorDiv(o.threadOrg[1]) +
+                         (warpId.floorDiv(o.warpOrg[1]) + d(3) * o.warpOrg[0]) * o.threadOrg[0];
+    return {4, {d(2), m * w}};
+  }
+  if (id == "loadFragB") {
+    const AffineExpr n = laneId % o.threadOrg[1] + (warpId % o.warpOrg[1] + d(3) * o.warpOrg[1]) * o.threadOrg[1];
+    return {4, {d(2), n * w}};
+  }
+  if (id == "cacheReadA" || id == "cacheReadB") return {1, {d(0)}};
+  if (id == "cacheWriteC") {
+    // operands: threadIdx.y, threadIdx.x, blockIdx.y, blockIdx.x, mi outer, ni outer, mi inner, ni inner
+    const AffineExpr m = laneId.floorDiv(o.threadOrg[1]) +
+                         (warpId.floorDiv(o.warpOrg[1]) + d(4).floorDiv(w) * o.warpOrg[0]) * o.threadOrg[0];
+    const AffineExpr n = laneId % o.threadOrg[1] +
+                         (warpId % o.warpOrg[1] + d(5).floorDiv(w) * o.warpOrg[1]) * o.threadOrg[1];
+    return {8, {d(2) * o.bm + m * w + d(6), d(3) * o.bn + n * w + d(7)}};
+  }
+  std::cerr << "getAffineMap: unknown map \"" << id << "\"\n";
+  return {};
+}
+
 void MatmulOptimizer::applyOptimzer(ModuleOp &module) {
   auto cfg = [&](const char *key, int fallback) {
     auto it = matmulConfig.find(key);
@@ -112,21 +210,140 @@ void MatmulOptimizer::applyOptimzer(ModuleOp &module) {
     DUMP(module);
 
     std::vector<ForOp> kmn_axes{loopK, m_inner, n_inner};
-    Rewriter::bufferizeLoopCarryVar(kmn_axes);  // tileC: THREAD_SIZE_M x THREAD_SIZE_N registers
+    Value tileC = Rewriter::bufferizeLoopCarryVar(kmn_axes);  // THREAD_SIZE_M x THREAD_SIZE_N registers
     DUMP(module);
 
     Rewriter::reorder({loopK, m_inner, n_inner});
     DUMP(module);
 
-    Rewriter::split(loopK, 2, {bk});
+    auto k_axes = Rewriter::split(loopK, 2, {bk});
     DUMP(module);
+
+    const int detail = cfg("SCHEDULE_DETAIL", 0);
+    const ThreadOrg org = threadOrg(matmulConfig);
+    if (detail >= 1 && !org.consistent)
+      std::cerr << "MatmulOptimizer: the staged schedule needs BLOCK_SIZE = 16 x THREAD_SIZE and whole warps; "
+                   "keeping the tiled nest\n";
+    if (detail >= 1 && org.consistent && k_axes.size() == 2) {
+      ForOp k_outer = k_axes[0], k_inner = k_axes[1];
+      const int width = static_cast<int>(org.width);
+      const MemoryBuffer &buf = matmulBuffers[matmul];
+      const DType elemA = buf.A.getMemRefType().elem, elemB = buf.B.getMemRefType().elem;
+
+      Value fragB = Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {org.fragB}, elemB);
+      Value fragA = Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {org.fragA}, elemA);
+      Value tileB = Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {org.ldgB}, elemB);
+      Value tileA = Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {org.ldgA}, elemA);
+      Value smB = Rewriter::alloc_buffer(OpHandle(gridLevel.op), MemorySpace::shared, {org.bk, org.bn}, elemB);
+      Value smA = Rewriter::alloc_buffer(OpHandle(gridLevel.op), MemorySpace::shared, {org.bk, org.bm}, elemA);
+      DUMP(module);
+
+      auto blockIdx = Rewriter::getParallelIdx(gridLevel);
+      auto threadIdx = Rewriter::getParallelIdx(blockLevel);
+
+      // global -> registers -> shared, once per k_outer step, fenced by two barriers
+      ForOp loadTileA = Rewriter::read(buf.A, tileA, getAffineMap("loadTileA"),
+                                       {threadIdx[0], threadIdx[1], blockIdx[0], k_outer.getInductionVar()}, width,
+                                       k_outer, Position::begin);
+      ForOp loadTileB = Rewriter::read(buf.B, tileB, getAffineMap("loadTileB"),
+                                       {threadIdx[0], threadIdx[1], k_outer.getInductionVar(), blockIdx[1]}, width,
+                                       loadTileA, Position::after);
+      DUMP(module);
+      ForOp storeTileA = Rewriter::write(tileA, smA, getAffineMap("storeTileA"), {threadIdx[0], threadIdx[1]}, width,
+                                         loadTileB, Position::after);
+      ForOp storeTileB = Rewriter::write(tileB, smB, getAffineMap("storeTileB"), {threadIdx[0], threadIdx[1]}, width,
+                                         storeTileA, Position::after);
+      Op *barrierPrefix = Rewriter::barrier(loadTileA, Position::before);
+      Op *barrierSuffix = Rewriter::barrier(storeTileB, Position::after);
+      DUMP(module);
+
+      // shared -> register fragments, once per k_inner step
+      ForOp loadFragA = Rewriter::read(smA, fragA, getAffineMap("loadFragA"),
+                                       {threadIdx[0], threadIdx[1], k_inner.getInductionVar()}, width, k_inner,
+                                       Position::begin);
+      ForOp loadFragB = Rewriter::read(smB, fragB, getAffineMap("loadFragB"),
+                                       {threadIdx[0], threadIdx[1], k_inner.getInductionVar()}, width, loadFragA,
+                                       Position::after);
+      DUMP(module);
+
+      Rewriter::cache_read(k_inner, buf.A, fragA, getAffineMap("cacheReadA"), {m_inner.getInductionVar()});
+      Rewriter::cache_read(k_inner, buf.B, fragB, getAffineMap("cacheReadB"), {n_inner.getInductionVar()});
+      DUMP(module);
+
+      // write-back of the register tile: width-wide vectors along n
+      auto writeC = Rewriter::get_write(blockLevel, buf.C);
+      if (writeC.size() == 1 && writeC[0].size() == 2) {
+        auto m_inner_axes = Rewriter::split(writeC[0][0], 2, {width});
+        auto n_inner_axes = Rewriter::split(writeC[0][1], 2, {width});
+        ForOp m_inner_0 = m_inner_axes[0], m_inner_1 = m_inner_axes[1];
+        ForOp n_inner_0 = n_inner_axes[0], n_inner_1 = n_inner_axes[1];
+        Rewriter::reorder({m_inner_0, n_inner_0, m_inner_1, n_inner_1});
+        DUMP(module);
+        Rewriter::cache_write(m_inner_0, buf.C, tileC, getAffineMap("cacheWriteC"),
+                              {threadIdx[0], threadIdx[1], blockIdx[0], blockIdx[1], m_inner_0.getInductionVar(),
+                               n_inner_0.getInductionVar(), m_inner_1.getInductionVar(),
+                               n_inner_1.getInductionVar()});
+        DUMP(module);
+        Rewriter::vectorize(n_inner_1, width);
+        DUMP(module);
+      } else {
+        std::cerr << "MatmulOptimizer: unexpected write-back nest, leaving it scalar\n";
+      }
+      matmul.setAttr("kcg.schedule", "staged");
+
+      if (detail >= 2) {
+        auto doubleLoadTileB = Rewriter::pipeline({loadTileB, storeTileB}, smB, k_outer);
+        auto doubleLoadTileA = Rewriter::pipeline({loadTileA, storeTileA}, smA, k_outer);
+        auto doubleLoadFragB = Rewriter::pipeline({loadFragB}, fragB, k_inner);
+        auto doubleLoadFragA = Rewriter::pipeline({loadFragA}, fragA, k_inner);
+        DUMP(module);
+
+        Rewriter::detach_last_loop(k_inner);
+        DUMP(module);
+
+        // prologue: A then B loads, A then B stores, one barrier
+        Rewriter::schedule(doubleLoadTileA[0][0].op, doubleLoadTileB[0][0].op, Position::before);
+        Rewriter::schedule(doubleLoadTileA[0][1].op, doubleLoadTileB[0][1].op, Position::before);
+        Rewriter::schedule(barrierPrefix, doubleLoadTileB[0][1].op, Position::after);
+        // main loop: global loads of the next slice first, its stores and the barrier after the k_inner loop
+        Rewriter::schedule(doubleLoadTileB[1][0].op, doubleLoadTileA[1][0].op, Position::after);
+        Rewriter::schedule(doubleLoadTileA[1][1].op, doubleLoadTileB[1][1].op, Position::before);
+        Rewriter::schedule(barrierSuffix, doubleLoadTileB[1][1].op, Position::after);
+        Op *ifOp = doubleLoadTileA[1][1]->parent;
+        Rewriter::schedule(ifOp, k_inner.op, Position::after);
+        // the first fragments of a slice are fetched before the slice's loop: once ahead of
+        // k_outer, and at the end of every k_outer step for the next one
+        Rewriter::extract_loop(doubleLoadFragA[0][0].op, k_outer, /*iteration*/ 0);
+        Rewriter::extract_loop(doubleLoadFragB[0][0].op, k_outer, /*iteration*/ 0);
+        Rewriter::schedule(doubleLoadFragB[0][0].op, k_outer.op, Position::end);
+        Rewriter::schedule(doubleLoadFragA[0][0].op, k_outer.op, Position::end);
+        DUMP(module);
+
+        Rewriter::change_double_buffer(doubleLoadFragA[0][0], smA);
+        Rewriter::change_double_buffer(doubleLoadFragB[0][0], smB);
+        DUMP(module);
+
+        Rewriter::take_off_true_if(module);
+        Rewriter::delete_false_if(module);
+        DUMP(module);
+
+        const int64_t threshold = std::max<int64_t>(bk, std::max(tm, tn));
+        Rewriter::unroll(module, [&](ForOp f) {
+          return f.tripCount() < std::min<int64_t>(threshold, width);
+        });
+        DUMP(module);
+        Rewriter::unrollAttribute(module, [&](ForOp f) { return f.tripCount() <= threshold; });
+        DUMP(module);
+        matmul.setAttr("kcg.schedule", "pipelined");
+      }
+    }
 
     Rewriter::unrollAttribute(module, 8);
 
     int64_t blockThreads = 0, gridBlocks = 0;
     Analyzer::getParallelNumber(blockLevel, blockThreads);
     Analyzer::getParallelNumber(gridLevel, gridBlocks);
-    matmul.setAttr("kcg.schedule", "tiled");
+    if (matmul.getAttr("kcg.schedule").empty()) matmul.setAttr("kcg.schedule", "tiled");
     matmul.setAttr("kcg.block_threads", std::to_string(blockThreads));
     matmul.setAttr("kcg.grid_blocks", std::to_string(gridBlocks));
   }

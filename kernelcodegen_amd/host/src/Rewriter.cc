@@ -1,5 +1,8 @@
 #include "Optimizer/Rewriter.h"
 
+#include <functional>
+#include <map>
+
 #include <algorithm>
 #include <iostream>
 #include <map>
@@ -331,6 +334,460 @@ ForOp Rewriter::outer_product(OpHandle where, Value tileC, Value fragA, Value fr
   Value add = append(lj.op, makeBinary(OpKind::AddF, mul, c))->result();
   append(lj.op, makeStore(add, tileC, {LinExpr(i), LinExpr(j)}));
   return li;
+}
+
+// ------------------------------------------------------------- staging
+namespace {
+
+Op *placeLoop(ForOp compute_at, Position pos, std::unique_ptr<Op> loop) {
+  switch (pos) {
+    case Position::before: return compute_at->insertBefore(std::move(loop));
+    case Position::after: return compute_at->insertAfter(std::move(loop));
+    case Position::begin: return compute_at->pushFront(std::move(loop));
+    case Position::end: return append(compute_at.op, std::move(loop));
+  }
+  return nullptr;
+}
+
+// body of a read loop: vector load src[map(operands, iv)], vector store dst[iv * width]
+void fillRead(Op *loop, Value src, Value dst, const AffineMap &map, std::vector<Value> operands, int64_t width) {
+  loop->pushBack(makeYield());
+  Op *yield = loop->lastOp();
+  operands.push_back(loop->arg(0));
+  Op *ld = yield->insertBefore(makeVectorLoad(src, {}, static_cast<int>(width)));
+  ld->indices = materialize(map, operands, ld);
+  LinExpr di;
+  di.add(loop->arg(0), width);
+  yield->insertBefore(makeVectorStore(ld->result(), dst, {di}, static_cast<int>(width)));
+}
+
+void fillWrite(Op *loop, Value src, Value dst, const AffineMap &map, std::vector<Value> operands, int64_t width) {
+  loop->pushBack(makeYield());
+  Op *yield = loop->lastOp();
+  const bool scatter = map.numDims - static_cast<int>(operands.size()) == 2;
+  operands.push_back(loop->arg(0));
+  if (!scatter) {
+    LinExpr si;
+    si.add(loop->arg(0), width);
+    Op *ld = yield->insertBefore(makeVectorLoad(src, {si}, static_cast<int>(width)));
+    Op *st = yield->insertBefore(makeVectorStore(ld->result(), dst, {}, static_cast<int>(width)));
+    st->indices = materialize(map, operands, st);
+    return;
+  }
+  Op *inner = yield->insertBefore(makeFor(0, width, 1));
+  inner->pushBack(makeYield());
+  Op *iy = inner->lastOp();
+  operands.push_back(inner->arg(0));
+  LinExpr si;
+  si.add(loop->arg(0), width);
+  si.add(inner->arg(0), 1);
+  Op *ld = iy->insertBefore(makeVectorLoad(src, {si}, 1));
+  Op *st = iy->insertBefore(makeVectorStore(ld->result(), dst, {}, 1));
+  st->indices = materialize(map, operands, st);
+}
+
+bool registerBuffer(Value v, const char *who) {
+  if (v && v.isMemRef() && v.getMemRefType().shape.size() == 1) return true;
+  std::cerr << who << ": the register-side buffer must be a one-dimensional memref\n";
+  return false;
+}
+
+}  // namespace
+
+ForOp Rewriter::read(Value src, Value dst, const AffineMap &map, std::vector<Value> operands, int64_t width,
+                     ForOp compute_at, Position pos) {
+  if (!registerBuffer(dst, "read") || width <= 0 || dst.getMemRefType().shape[0] % width != 0) return ForOp();
+  Op *loop = placeLoop(compute_at, pos, makeFor(0, dst.getMemRefType().shape[0] / width, 1));
+  fillRead(loop, src, dst, map, std::move(operands), width);
+  return ForOp(loop);
+}
+
+ForOp Rewriter::read(OpHandle where, Value src, Value dst, const AffineMap &map, std::vector<Value> operands,
+                     int64_t width) {
+  if (!registerBuffer(dst, "read") || width <= 0 || dst.getMemRefType().shape[0] % width != 0) return ForOp();
+  Op *loop = append(where.op, makeFor(0, dst.getMemRefType().shape[0] / width, 1));
+  fillRead(loop, src, dst, map, std::move(operands), width);
+  return ForOp(loop);
+}
+
+ForOp Rewriter::write(Value src, Value dst, const AffineMap &map, std::vector<Value> operands, int64_t width,
+                      ForOp compute_at, Position pos) {
+  if (!registerBuffer(src, "write") || width <= 0 || src.getMemRefType().shape[0] % width != 0) return ForOp();
+  Op *loop = placeLoop(compute_at, pos, makeFor(0, src.getMemRefType().shape[0] / width, 1));
+  fillWrite(loop, src, dst, map, std::move(operands), width);
+  return ForOp(loop);
+}
+
+ForOp Rewriter::write(OpHandle where, Value src, Value dst, const AffineMap &map, std::vector<Value> operands,
+                      int64_t width) {
+  if (!registerBuffer(src, "write") || width <= 0 || src.getMemRefType().shape[0] % width != 0) return ForOp();
+  Op *loop = append(where.op, makeFor(0, src.getMemRefType().shape[0] / width, 1));
+  fillWrite(loop, src, dst, map, std::move(operands), width);
+  return ForOp(loop);
+}
+
+void Rewriter::cache_read(ForOp scope, Value src, Value cached, const AffineMap &map,
+                          const std::vector<Value> &operands) {
+  std::vector<Op *> loads;
+  walk(scope.op, [&](Op *op) {
+    if (op->kind == OpKind::Load && op->vec == 0 && op->memref == src) loads.push_back(op);
+  });
+  for (Op *ld : loads) {
+    ld->memref = cached;
+    ld->indices = materialize(map, operands, ld);
+  }
+}
+
+void Rewriter::cache_write(ForOp scope, Value src, Value cached, const AffineMap &map,
+                           const std::vector<Value> &operands) {
+  (void)cached;
+  std::vector<Op *> stores;
+  walk(scope.op, [&](Op *op) {
+    if (op->kind == OpKind::Store && op->vec == 0 && op->memref == src) stores.push_back(op);
+  });
+  for (Op *st : stores) st->indices = materialize(map, operands, st);
+}
+
+std::vector<std::vector<ForOp>> Rewriter::get_write(ParallelOp parallelLevel, Value dst) {
+  std::vector<std::vector<ForOp>> results;
+  walk(parallelLevel.op, [&](Op *op) {
+    if (op->kind != OpKind::Store || op->memref != dst) return;
+    std::vector<ForOp> loops;
+    for (Op *p = op->parent; p && p != parallelLevel.op && p->kind == OpKind::For; p = p->parent)
+      loops.insert(loops.begin(), ForOp(p));
+    results.push_back(loops);
+  });
+  return results;
+}
+
+ForOp Rewriter::vectorize(ForOp readOrWrite, int64_t width) {
+  Op *l = readOrWrite.op;
+  if (!l || l->lb != 0 || l->step != 1 || width <= 0 || l->ub % width != 0) {
+    std::cerr << "vectorize: the loop must run from 0 in steps of 1 over a multiple of the width\n";
+    return ForOp();
+  }
+  l->step = width;
+  walk(l, [&](Op *op) {
+    if (op->kind == OpKind::Load) {
+      op->vec = static_cast<int>(width);
+      op->results[0]->lanes = static_cast<int>(width);
+    } else if (op->kind == OpKind::Store) {
+      op->vec = static_cast<int>(width);
+    }
+  });
+  return readOrWrite;
+}
+
+// ------------------------------------------------- pipelining
+namespace {
+
+// prepends a subscript to every access of `from` under `root` and retargets it to `to`
+void retarget(Op *root, Value from, Value to, const std::function<LinExpr(Op *)> &leading) {
+  std::vector<Op *> hits;
+  walk(root, [&](Op *op) {
+    if ((op->kind == OpKind::Load || op->kind == OpKind::Store) && op->memref == from) hits.push_back(op);
+  });
+  for (Op *op : hits) {
+    const LinExpr first = leading(op);
+    op->memref = to;
+    op->indices.insert(op->indices.begin(), first);
+  }
+}
+
+// affine.apply ops whose expression has become a constant (after an induction variable was
+// fixed) are folded into the expressions that use them
+void foldConstantApplies(Op *root) {
+  for (bool changed = true; changed;) {
+    changed = false;
+    std::vector<Op *> constant;
+    walk(root, [&](Op *op) {
+      if (op->kind == OpKind::Apply && op->indices[0].terms.empty()) constant.push_back(op);
+    });
+    for (Op *a : constant) {
+      int64_t v = a->indices[0].constant;
+      if (a->divisor > 0) {
+        int64_t q = v / a->divisor, r = v % a->divisor;
+        if (r < 0) {
+          r += a->divisor;
+          q -= 1;
+        }
+        v = a->isMod ? r : q;
+      }
+      Op *scope = a->parent;
+      replaceIndexUses(scope, a->result(), LinExpr(v));
+      a->erase();
+      changed = true;
+    }
+  }
+}
+
+// (iv floordiv step + offset) mod 2 as an index value computed right before `user`
+LinExpr halfSelector(Op *user, Value iv, int64_t step, int64_t offset) {
+  LinExpr q(iv);
+  if (step != 1) q = LinExpr(user->insertBefore(makeApplyFloorDiv(LinExpr(iv), step))->result());
+  q.constant += offset;
+  return LinExpr(user->insertBefore(makeApplyMod(q, 2))->result());
+}
+
+}  // namespace
+
+std::vector<std::vector<ForOp>> Rewriter::pipeline(std::vector<ForOp> readBodys, Value &buffer, ForOp compute_at) {
+  std::vector<std::vector<ForOp>> results;
+  Op *def = buffer ? buffer.getDefiningOp() : nullptr;
+  if (!def || def->kind != OpKind::Alloc || readBodys.empty()) {
+    std::cerr << "pipeline: the buffer must come from memref.alloc and there must be a loop that fills it\n";
+    return results;
+  }
+  for (auto r : readBodys)
+    if (!compute_at->isAncestorOf(r.op)) {
+      std::cerr << "pipeline: the filling loops must be inside the loop they are pipelined along\n";
+      return results;
+    }
+  Op *loop = compute_at.op;
+  Value iv = compute_at.getInductionVar();
+  const int64_t step = loop->step, lb = loop->lb, ub = loop->ub;
+
+  // 1. the double buffer
+  MemRefType t = buffer.getMemRefType();
+  t.shape.insert(t.shape.begin(), 2);
+  Value twice = def->insertBefore(makeAlloc(t))->result();
+
+  // 2. prologue: copies for the first iteration, into half 0
+  std::vector<ForOp> prologue;
+  for (auto r : readBodys) {
+    Op *copy = loop->insertBefore(clone(r.op));
+    replaceIndexUses(copy, iv, LinExpr(lb));
+    retarget(copy, buffer, twice, [](Op *) { return LinExpr(int64_t{0}); });
+    foldConstantApplies(copy);
+    prologue.emplace_back(copy);
+  }
+  results.push_back(prologue);
+  results.push_back(readBodys);
+
+  // 3. in the loop: fetch for the next iteration while there is one
+  LinExpr guard;  // ub - 2 * step - iv >= 0
+  guard.add(iv, -1);
+  guard.constant = ub - 2 * step;
+  Op *ifOp = loop->pushFront(makeIf({guard}));
+  for (auto r : readBodys) {
+    auto owned = r->unlink();
+    Op *moved = ifOp->pushBack(std::move(owned));
+    LinExpr next(iv);
+    next.constant = step;
+    replaceIndexUses(moved, iv, next);
+    retarget(moved, buffer, twice, [&](Op *user) { return halfSelector(user, iv, step, 1); });
+  }
+
+  // 4. every remaining access reads the half of the current iteration
+  Op *scope = def->parent;
+  retarget(scope, buffer, twice, [&](Op *user) { return halfSelector(user, iv, step, 0); });
+
+  def->erase();
+  buffer = twice;
+  return results;
+}
+
+void Rewriter::change_double_buffer(ForOp forOp, Value buffer) {
+  // the leading subscript of an access selects the half: flip it
+  walk(forOp.op, [&](Op *op) {
+    if ((op->kind != OpKind::Load && op->kind != OpKind::Store) || op->memref != buffer) return;
+    LinExpr &sel = op->indices[0];
+    if (sel.terms.empty()) {
+      sel.constant = 1 - sel.constant;
+      return;
+    }
+    // (x) mod 2 becomes (x + 1) mod 2
+    Op *def = sel.terms.size() == 1 && sel.terms[0].second == 1 && sel.constant == 0
+                  ? sel.terms[0].first.getDefiningOp()
+                  : nullptr;
+    if (def && def->kind == OpKind::Apply && def->isMod && def->divisor == 2) {
+      LinExpr inner = def->indices[0];
+      inner.constant += 1;
+      sel = LinExpr(op->insertBefore(makeApplyMod(inner, 2))->result());
+      return;
+    }
+    // any other 0/1 selector s: 1 - s
+    LinExpr flipped(int64_t{1});
+    flipped.add(sel, -1);
+    sel = flipped;
+  });
+}
+
+void Rewriter::detach_last_loop(ForOp forOp) {
+  Op *l = forOp.op;
+  if (l->args.size() != 1 || l->ub - l->step < l->lb) {
+    std::cerr << "detach_last_loop: needs a loop without iter_args and at least one iteration\n";
+    return;
+  }
+  const int64_t last = l->ub - l->step;
+  l->ub = last;
+  std::map<ValueImpl *, ValueImpl *> mapping;
+  auto copy = clone(l, &mapping);
+  Value copyIv = copy->arg(0);
+  replaceIndexUses(copy.get(), copyIv, LinExpr(last));
+  foldConstantApplies(copy.get());
+  copy->body.pop_back();  // the terminator
+  Op *after = l;
+  while (!copy->body.empty()) {
+    std::unique_ptr<Op> k = std::move(copy->body.front());
+    copy->body.pop_front();
+    after = after->insertAfter(std::move(k));
+  }
+}
+
+void Rewriter::schedule(Op *srcOp, Op *dstOp, Position pos) {
+  switch (pos) {
+    case Position::after: srcOp->moveAfter(dstOp); break;
+    case Position::before: srcOp->moveBefore(dstOp); break;
+    case Position::end:
+      if (dstOp->kind == OpKind::For) srcOp->moveBefore(dstOp->lastOp());
+      else std::cerr << "schedule: Position::end needs a loop as destination\n";
+      break;
+    default: std::cerr << "schedule: Position::begin is not supported\n"; break;
+  }
+}
+
+Op *Rewriter::extract_loop(Op *srcOp, ForOp forOp, int64_t iteration) {
+  Op *copy = forOp->insertBefore(clone(srcOp));
+  replaceIndexUses(copy, forOp.getInductionVar(), LinExpr(forOp->lb + iteration * forOp->step));
+  foldConstantApplies(copy);
+  return copy;
+}
+
+// ------------------------------------------------------------ clean-up
+namespace {
+
+// value range of an index value: loop / parallel induction variables and
+// floordiv / mod / linear applies of ranged values
+bool rangeOf(Value v, int64_t &lo, int64_t &hi);
+
+bool rangeOf(const LinExpr &e, int64_t &lo, int64_t &hi) {
+  lo = hi = e.constant;
+  for (auto &t : e.terms) {
+    int64_t a, b;
+    if (!rangeOf(t.first, a, b)) return false;
+    if (t.second >= 0) {
+      lo += a * t.second;
+      hi += b * t.second;
+    } else {
+      lo += b * t.second;
+      hi += a * t.second;
+    }
+  }
+  return true;
+}
+
+int64_t floorDivide(int64_t a, int64_t c) {
+  int64_t q = a / c;
+  if (a % c != 0 && a < 0) --q;
+  return q;
+}
+
+bool rangeOf(Value v, int64_t &lo, int64_t &hi) {
+  ValueImpl *impl = v.get();
+  if (!impl) return false;
+  if (impl->kind == ValueImpl::InductionVar) {
+    Op *o = impl->owner;
+    if (o->kind == OpKind::For) {
+      if (o->ub <= o->lb) return false;
+      lo = o->lb;
+      hi = o->lb + (ForOp(o).tripCount() - 1) * o->step;
+      return true;
+    }
+    if (o->kind == OpKind::Parallel) {
+      lo = 0;
+      hi = o->ubs[impl->index] - 1;
+      return true;
+    }
+    return false;
+  }
+  Op *def = v.getDefiningOp();
+  if (!def || def->kind != OpKind::Apply) return false;
+  int64_t a, b;
+  if (!rangeOf(def->indices[0], a, b)) return false;
+  if (def->divisor == 0) {
+    lo = a;
+    hi = b;
+  } else if (!def->isMod) {
+    lo = floorDivide(a, def->divisor);
+    hi = floorDivide(b, def->divisor);
+  } else if (floorDivide(a, def->divisor) == floorDivide(b, def->divisor)) {
+    lo = a - floorDivide(a, def->divisor) * def->divisor;
+    hi = b - floorDivide(b, def->divisor) * def->divisor;
+  } else {
+    lo = 0;
+    hi = def->divisor - 1;
+  }
+  return true;
+}
+
+// +1: every constraint always holds; -1: some constraint never holds; 0: undecided
+int decide(Op *ifOp) {
+  bool allTrue = true;
+  for (auto &c : ifOp->indices) {
+    int64_t lo, hi;
+    if (!rangeOf(c, lo, hi)) return 0;
+    if (hi < 0) return -1;
+    if (lo < 0) allTrue = false;
+  }
+  return allTrue ? 1 : 0;
+}
+
+std::vector<Op *> collectIfs(Op *root) {
+  std::vector<Op *> ifs;
+  walk(root, [&](Op *op) {
+    if (op->kind == OpKind::If) ifs.push_back(op);
+  }, WalkOrder::PostOrder);
+  return ifs;
+}
+
+}  // namespace
+
+void Rewriter::take_off_true_if(ModuleOp module) {
+  for (Op *ifOp : collectIfs(module.get())) {
+    if (decide(ifOp) != 1) continue;
+    Op *after = ifOp;
+    while (!ifOp->body.empty()) {
+      std::unique_ptr<Op> k = std::move(ifOp->body.front());
+      ifOp->body.pop_front();
+      if (k->kind == OpKind::Yield) continue;
+      after = after->insertAfter(std::move(k));
+    }
+    ifOp->erase();
+  }
+}
+
+void Rewriter::delete_false_if(ModuleOp module) {
+  for (Op *ifOp : collectIfs(module.get()))
+    if (decide(ifOp) == -1) ifOp->erase();
+}
+
+void Rewriter::unroll(ModuleOp module, const std::function<bool(ForOp)> &unrollCheckFn) {
+  std::vector<Op *> loops;
+  walk(module.get(), [&](Op *op) {
+    if (op->kind == OpKind::For && op->args.size() == 1 && unrollCheckFn(ForOp(op))) loops.push_back(op);
+  }, WalkOrder::PostOrder);
+  for (Op *l : loops) {
+    Op *after = l;
+    for (int64_t iv = l->lb; iv < l->ub; iv += l->step) {
+      auto copy = clone(l);
+      replaceIndexUses(copy.get(), copy->arg(0), LinExpr(iv));
+      foldConstantApplies(copy.get());
+      copy->body.pop_back();
+      while (!copy->body.empty()) {
+        std::unique_ptr<Op> k = std::move(copy->body.front());
+        copy->body.pop_front();
+        after = after->insertAfter(std::move(k));
+      }
+    }
+    l->erase();
+  }
+}
+
+void Rewriter::unrollAttribute(ModuleOp module, const std::function<bool(ForOp)> &unrollCheckFn) {
+  walk(module.get(), [&](Op *op) {
+    if (op->kind == OpKind::For && unrollCheckFn(ForOp(op))) op->attrs["affine.loop"] = "unroll";
+  });
 }
 
 void Rewriter::unrollAttribute(ModuleOp module, int64_t maxTrips) {

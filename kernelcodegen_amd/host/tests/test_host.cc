@@ -32,6 +32,12 @@ static int g_failed = 0, g_checks = 0;
     }                                                                            \
   } while (0)
 
+static int count(const std::string &hay, const std::string &needle) {
+  int n = 0;
+  for (size_t pos = hay.find(needle); pos != std::string::npos; pos = hay.find(needle, pos + 1)) ++n;
+  return n;
+}
+
 static bool contains(const std::string &hay, const std::string &needle) {
   return hay.find(needle) != std::string::npos;
 }
@@ -255,6 +261,92 @@ static void test_schedule_preserves_results() {
     CHECK(std::memcmp(c.data(), expect.data(), c.size() * sizeof(float)) == 0);
     CHECK(interp.buffer(f.C) == c.data());   // the call result aliases the C buffer
   }
+}
+
+// The staged (SCHEDULE_DETAIL 1) and pipelined (2) schedules of the reference recipe
+// (src/Optimizer/Optimizer.cc:429-546), run by the interpreter with the threads of
+// a block in lock step: results must equal the naive nest bit for bit, for the
+// reference's 32-wide warps and for 64-wide waves.
+static void run_detailed_schedule(int detail, int warp, int64_t M, int64_t N, int64_t K, int bk, std::string *text) {
+  std::vector<float> a(M * K), b(K * N);
+  unsigned s = 777u + detail + warp;
+  auto rnd = [&]() {
+    s = s * 1664525u + 1013904223u;
+    return static_cast<float>(static_cast<int>(s >> 8) % 2001 - 1000) / 512.0f;
+  };
+  for (auto &x : a) x = rnd();
+  for (auto &x : b) x = rnd();
+  std::vector<float> expect(M * N);
+  for (int64_t i = 0; i < M; ++i)
+    for (int64_t j = 0; j < N; ++j) {
+      float acc = 0.0f;
+      for (int64_t k = 0; k < K; ++k) {
+        volatile float mul = a[i * K + k] * b[k * N + j];
+        acc = mul + acc;
+      }
+      expect[i * N + j] = acc;
+    }
+  MatmulFixture f(M, N, K);
+  MatmulOptimizer opt;
+  MatmulOptimizer::matmulConfig = {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", bk},
+                                   {"THREAD_SIZE_M", 8},  {"THREAD_SIZE_N", 8},   {"VECTORIZE_WIDTH", 4},
+                                   {"WARP_SIZE", warp},   {"SCHEDULE_DETAIL", detail}};
+  CHECK(opt.applicable(f.graph->module));
+  opt.applyOptimzer(f.graph->module);
+  const std::string problem = verify(f.graph->module.get());
+  CHECK(problem.empty());
+  if (!problem.empty()) std::fprintf(stderr, "    verify: %s\n", problem.c_str());
+  CHECK(f.func.getAttr("kcg.schedule") == (detail == 1 ? "staged" : "pipelined"));
+  if (text) *text = f.graph->module.str();
+  std::vector<float> c(M * N, -1.0f);
+  Interpreter interp(f.graph->module);
+  interp.bind(f.A, a.data());
+  interp.bind(f.B, b.data());
+  Value cbuf = Analyzer::collectFuncCalls(f.graph->module)[0].getArgOperands()[2];
+  interp.bind(cbuf, c.data());
+  const std::string err = interp.run();
+  CHECK(err.empty());
+  if (!err.empty()) std::fprintf(stderr, "    interpreter: %s\n", err.c_str());
+  CHECK(std::memcmp(c.data(), expect.data(), c.size() * sizeof(float)) == 0);
+}
+
+static void test_staged_schedule() {
+  std::string text;
+  run_detailed_schedule(1, 32, 128, 256, 24, 8, &text);
+  // README stage "read / write / barrier / cache_read / cache_write / vectorize" facts
+  CHECK(contains(text, "memref<8x128xf32, 2>"));            // smA, smB: BLOCK_SIZE_K x 128
+  CHECK(contains(text, "memref<4xf32, 3>"));                // tileA / tileB: 8*128/256 registers
+  CHECK(contains(text, "memref<8xf32, 3>"));                // fragA / fragB
+  CHECK(count(text, "gpu.barrier") == 2);
+  CHECK(count(text, "affine.vector_load %arg0[") == 1);     // one global read loop per operand
+  CHECK(count(text, "affine.vector_load %arg1[") == 1);
+  CHECK(contains(text, "floordiv 2"));                      // thread id -> (row, 4-wide k chunk) of the A tile
+  CHECK(contains(text, "floordiv 32"));                     // thread id -> (k row, 4-wide n chunk) of the B tile
+  CHECK(contains(text, ", vector<1xf32>"));                 // transposing store of A, element by element
+  CHECK(contains(text, "memref<128x256xf32, 1>, vector<4xf32>"));   // C written as float4
+  CHECK(!contains(text, "affine.load %arg0[") && !contains(text, "affine.load %arg1["));   // operands come from fragments
+  run_detailed_schedule(1, 64, 256, 128, 16, 8, nullptr);
+  run_detailed_schedule(1, 64, 128, 128, 32, 16, nullptr);
+}
+
+static void test_pipelined_schedule() {
+  std::string text;
+  run_detailed_schedule(2, 32, 128, 256, 32, 8, &text);
+  // README final-stage facts: double-buffered shared tiles and fragments, the guard of the
+  // in-loop prefetch, no always-true / never-true affine.if left
+  CHECK(contains(text, "memref<2x8x128xf32, 2>"));
+  CHECK(contains(text, "memref<2x8xf32, 3>"));
+  CHECK(!contains(text, "memref<8x128xf32, 2>"));
+  CHECK(contains(text, "affine.if affine_set<(d0) : (-d0 + 16 >= 0)>"));   // k_outer + 2*8 <= 32
+  // one guard around the global loads of the next slice (top of the k_outer body), one around
+  // its stores to shared memory and the barrier (after the k_inner loop); the guards along
+  // k_inner were decided statically and are gone
+  CHECK(count(text, "affine.if") == 2);
+  CHECK(!contains(text, "(0) floordiv") && !contains(text, "(7) mod"));   // constants are folded
+  CHECK(contains(text, "mod 2"));
+  CHECK(contains(text, "affine.loop = \"unroll\""));
+  run_detailed_schedule(2, 64, 256, 128, 48, 8, nullptr);
+  run_detailed_schedule(2, 64, 128, 128, 64, 16, nullptr);
 }
 
 static void test_relu_softmax_batched_matmul_semantics() {
@@ -684,6 +776,8 @@ int main() {
       {"frontend_matmul_nest", test_frontend_matmul_nest},
       {"schedule_stages_match_readme", test_schedule_stages_match_readme},
       {"schedule_preserves_results", test_schedule_preserves_results},
+      {"staged_schedule", test_staged_schedule},
+      {"pipelined_schedule", test_pipelined_schedule},
       {"relu_softmax_batched_matmul_semantics", test_relu_softmax_batched_matmul_semantics},
       {"batched_matmul_layouts", test_batched_matmul_layouts},
       {"fmha_pattern_and_fusion", test_fmha_pattern_and_fusion},
