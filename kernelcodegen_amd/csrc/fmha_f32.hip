@@ -8,7 +8,7 @@
 // The tiling idea is kept (a workgroup owns Br query rows and sweeps K/V in Bc
 // row tiles, running max / sum / rescale).  Everything else is gfx950 specific:
 //
-//  * 4 waves per workgroup, 32 query rows per wave, Br = 128, Bc = 32 (or 64).
+//  * 4 (or 8) waves per workgroup, 32 query rows per wave, Br = 128 (256), Bc = 32 (or 64).
 //  * The first product is computed transposed, S^T = K . Q^T, with
 //    v_mfma_f32_32x32x2_f32: lane (r = l%32, h = l/32) then holds, for query r,
 //    the 16 keys {8g + 4h + i}.  That is exactly the B-operand layout the second
@@ -20,6 +20,11 @@
 //  * K and V tiles are staged in padded LDS in their global layout; the next
 //    tile's global loads are issued before the MFMA phase that hides them
 //    (V_t during S = K_t.Q, K_{t+1} during O += P.V_t).
+//  * The running maximum is a lazily raised reference (see kTau): VALU work between
+//    the two MFMA phases costs matrix time, so the rescale of O is skipped whenever
+//    the mathematics allows it.
+//  * Causal: a workgroup runs the query-block pair (n-1-i, i), so all workgroups
+//    sweep the same number of tiles.
 //
 // LDS (floats): Ks[Bc][D+4]  (b128 reads of 16 consecutive rows hit 64 banks)
 //               Vs[Bc][D+8]  (rows 4 apart are 32 banks apart: the two halves of
@@ -28,10 +33,10 @@
 
 namespace kcg {
 
-template <int D, int BC>
+template <int D, int BC, int WAVES>
 struct FmhaF32Tile {
-  static constexpr int kThreads = 256;
-  static constexpr int kBr = 128;
+  static constexpr int kThreads = 64 * WAVES;
+  static constexpr int kBr = 32 * WAVES;
   static constexpr int kPitchK = D + 4;
   static constexpr int kPitchV = D + 8;
   static constexpr int kLdsBytes = (BC * kPitchK + BC * kPitchV) * 4;
@@ -42,25 +47,49 @@ struct FmhaF32Tile {
   static_assert((BC * D / 4) % kThreads == 0, "load split");
 };
 
-template <int D, int BC, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restrict__ Q,
+// How far (in log2 units) a tile's row maximum may exceed the running reference before
+// the accumulators are rescaled.
+constexpr float kTau = 8.0f;
+
+// v_max3_f32 without the canonicalising self-max the compiler puts in front of fmaxf on
+// MFMA results (NaN operands are ignored like in fmaxf; a NaN score still reaches the
+// output through its own exponential).
+__device__ __forceinline__ float max3(float a, float b, float c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+#else
+  return fmaxf(fmaxf(a, b), c);
+#endif
+}
+
+// max over both halves of the wave for the same lane%32 (one v_permlane32_swap)
+__device__ __forceinline__ float max_across_halves(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+
+template <int D, int BC, int WAVES, bool CAUSAL>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const float *__restrict__ Q,
                                                           const float *__restrict__ K,
                                                           const float *__restrict__ V,
                                                           float *__restrict__ O, int S,
-                                                          int q_blocks, float scale_log2e) {
-  using T = FmhaF32Tile<D, BC>;
+                                                          int q_blocks, int q_items, float scale_log2e) {
+  using T = FmhaF32Tile<D, BC, WAVES>;
   extern __shared__ __align__(16) float lds[];
   float *Ks = lds;
   float *Vs = lds + BC * T::kPitchK;
 
-  // Every XCD walks a contiguous range of (head, query block) ids, head-major, so
-  // the K/V of a head are fetched into one XCD's L2 only.  Heavy (late) query
-  // blocks first when causal, so the tail of the grid is cheap.
+  // Every XCD walks a contiguous range of (head, work item) ids, head-major, so the
+  // K/V of a head are fetched into one XCD's L2 only.  Causal: a work item is the pair
+  // of query blocks (n-1-i, i), so every workgroup sweeps the same number of K/V tiles.
   const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int bh = bid / q_blocks;
-  const int qb_raw = bid - bh * q_blocks;
-  const int qb = CAUSAL ? (q_blocks - 1 - qb_raw) : qb_raw;
-  const int q0 = qb * T::kBr;
+  const int bh = bid / q_items;
+  const int item = bid - bh * q_items;
+  const int hi_block = q_blocks - 1 - item;
+  const int npass = CAUSAL ? (hi_block != item ? 2 : 1) : 1;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -74,6 +103,42 @@ __global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restric
   const float *Vb = V + base;
   float *Ob = O + base;
 
+
+  // Tile transfer: thread -> (row ld_row + i * kRowsPerIter, 16-byte column ld_c4).  A full
+  // tile is fetched with a uniform base (scalar registers) plus one per-lane byte offset;
+  // only the ragged last tile pays for per-row predicates (rows at and beyond S read as 0).
+  constexpr int kRowsPerIter = T::kThreads / (D / 4);
+  const int ld_row = tid / (D / 4);
+  const int ld_c4 = tid % (D / 4);
+  const unsigned ld_off = static_cast<unsigned>(ld_row * D + ld_c4 * 4) * 4u;
+  float4_t stage[T::kLoads];
+  auto load_tile = [&](const float *src, int kv0) {
+    const char *g = reinterpret_cast<const char *>(src + static_cast<int64_t>(kv0) * D);
+    if (kv0 + BC <= S) {
+#pragma unroll
+      for (int i = 0; i < T::kLoads; ++i)
+        stage[i] = *reinterpret_cast<const float4_t *>(g + i * (kRowsPerIter * D * 4) + ld_off);
+    } else {
+#pragma unroll
+      for (int i = 0; i < T::kLoads; ++i) {
+        float4_t v = {0.f, 0.f, 0.f, 0.f};
+        if (kv0 + ld_row + i * kRowsPerIter < S)
+          v = *reinterpret_cast<const float4_t *>(g + i * (kRowsPerIter * D * 4) + ld_off);
+        stage[i] = v;
+      }
+    }
+  };
+  auto store_tile = [&](float *dst, int pitch) {
+    float *d = dst + ld_row * pitch + ld_c4 * 4;
+#pragma unroll
+    for (int i = 0; i < T::kLoads; ++i)
+      *reinterpret_cast<float4_t *>(d + i * kRowsPerIter * pitch) = stage[i];
+  };
+
+#pragma unroll 1
+  for (int pass = 0; pass < npass; ++pass) {
+  const int qb = CAUSAL ? (pass == 0 ? hi_block : item) : item;  // the long block first
+  const int q0 = qb * T::kBr;
   const int qrow = q0 + wave * 32 + r32;  // this lane's query
   const bool qvalid = qrow < S;
 
@@ -94,34 +159,11 @@ __global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restric
   for (int i = 0; i < T::kDTiles; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc_o[i][e] = 0.0f;
-  float m_run = -INFINITY;  // running max of this query (both halves agree)
+  float m_run = -INFINITY;  // reference max of this query (both halves agree)
   float l_run = 0.0f;       // running sum over this lane's keys only
 
   const int kv_end = CAUSAL ? ((q0 + T::kBr) < S ? (q0 + T::kBr) : S) : S;
   const int n_tiles = (kv_end + BC - 1) / BC;
-
-  float4_t stage[T::kLoads];
-  auto load_tile = [&](const float *src, int kv0) {
-#pragma unroll
-    for (int i = 0; i < T::kLoads; ++i) {
-      const int idx = tid + i * T::kThreads;
-      const int row = idx / (D / 4);
-      const int c4 = idx % (D / 4);
-      float4_t v = {0.f, 0.f, 0.f, 0.f};
-      if (kv0 + row < S)
-        v = *reinterpret_cast<const float4_t *>(src + static_cast<int64_t>(kv0 + row) * D + c4 * 4);
-      stage[i] = v;
-    }
-  };
-  auto store_tile = [&](float *dst, int pitch) {
-#pragma unroll
-    for (int i = 0; i < T::kLoads; ++i) {
-      const int idx = tid + i * T::kThreads;
-      const int row = idx / (D / 4);
-      const int c4 = idx % (D / 4);
-      *reinterpret_cast<float4_t *>(dst + row * pitch + c4 * 4) = stage[i];
-    }
-  };
 
   load_tile(Kb, 0);
   store_tile(Ks, T::kPitchK);
@@ -138,12 +180,18 @@ __global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restric
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[kt][e] = 0.0f;
       const float *kp = Ks + (kt * 32 + r32) * T::kPitchK + 4 * half;
+      // the K fragment of the next 8 d-columns is requested before the four MFMAs of the
+      // current one are issued
+      float4_t kf[2];
+      kf[0] = *reinterpret_cast<const float4_t *>(kp);
 #pragma unroll
       for (int kk = 0; kk < D / 8; ++kk) {
-        const float4_t kf = *reinterpret_cast<const float4_t *>(kp + 8 * kk);
+        if (kk + 1 < D / 8) kf[(kk + 1) & 1] = *reinterpret_cast<const float4_t *>(kp + 8 * (kk + 1));
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[j], q[kk][j], s[kt], 0, 0, 0);
+          s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[kk & 1][j], q[kk][j], s[kt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 
@@ -160,16 +208,27 @@ __global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restric
         }
     }
 
-    // ---- online softmax (base 2; Q carries scale * log2 e) ----
-    float m_loc = -INFINITY;
+    // ---- online softmax (base 2; Q carries scale * log2 e), lazy rescale ----
+    // m_run is a reference maximum, not the exact one: it is raised (and O, l rescaled)
+    // only when the tile maximum exceeds it by more than kTau, so that after the first
+    // tiles almost no tile pays the 16 * kDTiles multiplications.  Between rescales
+    // P <= 2^kTau; the final O / l is exact for any reference.  The decision is per
+    // query row (both lanes of a row see the same m_loc and m_run).
+    float m_loc = max3(s[0][0], s[0][1], s[0][2]);
 #pragma unroll
-    for (int kt = 0; kt < T::kKeyTiles; ++kt)
+    for (int x = 3; x + 1 < T::kKeyTiles * 16; x += 2) m_loc = max3(m_loc, s[x / 16][x % 16], s[(x + 1) / 16][(x + 1) % 16]);
+    m_loc = max_across_halves(fmaxf(m_loc, s[T::kKeyTiles - 1][15]));
+    const bool raise = m_loc > m_run + kTau;  // false for NaN and for rows masked so far
+    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+      const float alpha = raise ? __builtin_amdgcn_exp2f(m_run - m_loc) : 1.0f;  // m_run = -inf -> 0
+      if (raise) m_run = m_loc;
+      l_run *= alpha;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) m_loc = fmaxf(m_loc, s[kt][e]);
-    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
-    const float m_new = fmaxf(m_run, m_loc);
-    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;  // fully masked so far
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);                 // m_run = -inf -> 0
+      for (int i = 0; i < T::kDTiles; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc_o[i][e] *= alpha;
+    }
+    const float m_use = (m_run == -INFINITY) ? 0.0f : m_run;  // fully masked so far
     float psum = 0.0f;
 #pragma unroll
     for (int kt = 0; kt < T::kKeyTiles; ++kt)
@@ -179,12 +238,7 @@ __global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restric
         s[kt][e] = p;
         psum += p;
       }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-#pragma unroll
-    for (int i = 0; i < T::kDTiles; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc_o[i][e] *= alpha;
+    l_run += psum;
 
     store_tile(Vs, T::kPitchV);
     __syncthreads();  // V tile visible; every wave is done reading Ks
@@ -193,17 +247,33 @@ __global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restric
     if (more) load_tile(Kb, kv0 + BC);
 
     // ---- O^T += V^T . P^T  (rows = d, columns = queries, contraction over keys) ----
-#pragma unroll
-    for (int kt = 0; kt < T::kKeyTiles; ++kt) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
+    // The matrix phase with the longer dependency chains gets the higher wave priority:
+    // two workgroups sharing a CU then take turns instead of the older one always winning.
+    __builtin_amdgcn_s_setprio(1);
+    {
+      // step x = (kt, e): key 32*kt + 8*(e/4) + 4*half + e%4; its kDTiles V values are
+      // requested one step (kDTiles MFMAs) ahead
+      constexpr int kPvSteps = T::kKeyTiles * 16;
+      float vf[2][T::kDTiles];
+      auto vfetch = [&](int x) {
+        const int kt = x / 16, e = x % 16;
         const float *vp = Vs + (kt * 32 + 8 * (e / 4) + 4 * half + (e % 4)) * T::kPitchV + r32;
 #pragma unroll
+        for (int i = 0; i < T::kDTiles; ++i) vf[x & 1][i] = vp[i * 32];
+      };
+      vfetch(0);
+#pragma unroll
+      for (int x = 0; x < kPvSteps; ++x) {
+        if (x + 1 < kPvSteps) vfetch(x + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
         for (int i = 0; i < T::kDTiles; ++i)
-          acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(vp[i * 32], s[kt][e], acc_o[i], 0, 0, 0);
+          acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[x & 1][i], s[x / 16][x % 16], acc_o[i], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 
+    __builtin_amdgcn_s_setprio(0);
     if (more) store_tile(Ks, T::kPitchK);
     __syncthreads();  // next K tile visible; every wave is done reading Vs
   }
@@ -222,15 +292,17 @@ __global__ __launch_bounds__(256, 2) void fmha_f32_kernel(const float *__restric
         *reinterpret_cast<float4_t *>(Ob + static_cast<int64_t>(qrow) * D + 32 * i + 8 * g + 4 * half) = v;
       }
   }
+  }  // pass
 }
 
-template <int D, int BC>
+template <int D, int BC, int WAVES>
 static int launch_fmha_f32(const float *Q, const float *K, const float *V, float *O, int B, int H,
                            int S, float scale, int causal, hipStream_t stream,
                            kcg_launch_info *info) {
-  using T = FmhaF32Tile<D, BC>;
+  using T = FmhaF32Tile<D, BC, WAVES>;
   const int64_t q_blocks = (static_cast<int64_t>(S) + T::kBr - 1) / T::kBr;
-  const int64_t blocks = q_blocks * B * H;
+  const int64_t q_items = causal ? (q_blocks + 1) / 2 : q_blocks;
+  const int64_t blocks = q_items * B * H;
   if (blocks > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
   if (info) {
     info->grid[0] = static_cast<int>(blocks);
@@ -238,18 +310,19 @@ static int launch_fmha_f32(const float *Q, const float *K, const float *V, float
     info->block[0] = T::kThreads;
     info->block[1] = info->block[2] = 1;
     info->lds_bytes = T::kLdsBytes;
-    info->waves_per_block = 4;
+    info->waves_per_block = WAVES;
     snprintf(info->kernel, sizeof info->kernel, "fmha_f32_d%d_br%d_bc%d%s", D, T::kBr, BC,
-             causal ? "_causal" : "");
+             causal ? "_causal_paired" : "");
     return KCG_OK;
   }
   const float scale_log2e = scale * 1.4426950408889634f;
 #define KCG_LAUNCH(CAUSAL_)                                                                       \
   do {                                                                                            \
-    auto kern = fmha_f32_kernel<D, BC, CAUSAL_>;                                                  \
+    auto kern = fmha_f32_kernel<D, BC, WAVES, CAUSAL_>;                                                  \
     if (!allow_lds(kern, T::kLdsBytes)) return KCG_ERR_LAUNCH;                                    \
     return launch(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads), T::kLdsBytes,     \
-                  stream, Q, K, V, O, S, static_cast<int>(q_blocks), scale_log2e);                \
+                  stream, Q, K, V, O, S, static_cast<int>(q_blocks), static_cast<int>(q_items),     \
+                  scale_log2e);                \
   } while (0)
   if (causal) KCG_LAUNCH(true);
   else KCG_LAUNCH(false);
@@ -264,17 +337,20 @@ int dispatch_fmha_f32(const float *Q, const float *K, const float *V, float *O, 
     if (sched->br) br = sched->br;
     if (sched->bc) bc = sched->bc;
   }
-  if (br != 128) return KCG_ERR_BAD_SCHEDULE;
-  if (D == 128) {
-    if (bc == 64) return launch_fmha_f32<128, 64>(Q, K, V, O, B, H, S, scale, causal, stream, info);
-    if (bc == 32) return launch_fmha_f32<128, 32>(Q, K, V, O, B, H, S, scale, causal, stream, info);
-    return KCG_ERR_BAD_SCHEDULE;
-  }
-  if (D == 64) {
-    if (bc == 64) return launch_fmha_f32<64, 64>(Q, K, V, O, B, H, S, scale, causal, stream, info);
-    if (bc == 32) return launch_fmha_f32<64, 32>(Q, K, V, O, B, H, S, scale, causal, stream, info);
-    return KCG_ERR_BAD_SCHEDULE;
-  }
+  if (br != 128 && br != 256) return KCG_ERR_BAD_SCHEDULE;
+  if (bc != 32 && bc != 64) return KCG_ERR_BAD_SCHEDULE;
+#define KCG_PICK(D_, BC_, WAVES_)                \
+  if (D == D_ && bc == BC_ && br == 32 * WAVES_) \
+    return launch_fmha_f32<D_, BC_, WAVES_>(Q, K, V, O, B, H, S, scale, causal, stream, info);
+  KCG_PICK(128, 32, 4)
+  KCG_PICK(128, 32, 8)
+  KCG_PICK(128, 64, 4)
+  KCG_PICK(64, 32, 4)
+  KCG_PICK(64, 32, 8)
+  KCG_PICK(64, 64, 4)
+  KCG_PICK(64, 64, 8)
+#undef KCG_PICK
+  if (D == 128 || D == 64) return KCG_ERR_BAD_SCHEDULE;
   return KCG_ERR_UNSUPPORTED_SHAPE;
 }
 

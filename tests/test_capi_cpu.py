@@ -88,6 +88,14 @@ def test_launch_geometry_queries():
     assert info.grid[0] == 4 * 32 * 32 and info.lds_bytes == 2 * 2 * 64 * 128 * 2
     assert L.kcg_fmha_query(0, 1, 32, 2048, 128, 0, None, ctypes.byref(info)) == 0
     assert info.grid[0] == 32 * 2048 // 128
+    # fp32 causal: 128-row query blocks in pairs; the 8-wave workgroup is a schedule option
+    assert L.kcg_fmha_query(0, 1, 32, 2048, 128, 1, None, ctypes.byref(info)) == 0
+    assert info.grid[0] == 32 * 8 and b"causal_paired" in info.kernel
+    s256 = lib.FmhaSched(br=256, bc=32)
+    assert L.kcg_fmha_query(0, 1, 32, 2048, 128, 0, ctypes.byref(s256), ctypes.byref(info)) == 0
+    assert info.grid[0] == 32 * 8 and info.block[0] == 512 and info.waves_per_block == 8
+    s256.bc = 64
+    assert L.kcg_fmha_query(0, 1, 32, 2048, 128, 0, ctypes.byref(s256), ctypes.byref(info)) == 4
     assert L.kcg_fmha_query(7, 1, 1, 128, 128, 0, None, ctypes.byref(info)) == 5
     assert L.kcg_fmha_query(0, 1, 1, 128, 80, 0, None, ctypes.byref(info)) == 3
 

@@ -32,16 +32,41 @@ SHAPES = [(1, 2, 128, 128), (1, 2, 256, 64), (2, 3, 200, 128), (1, 1, 77, 64), (
 
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("bc", [32, 64])
-def test_f32_parity(oracle, dev, shape, causal, bc):
+@pytest.mark.parametrize("tile", [(128, 32), (128, 64), (256, 32)])
+def test_f32_parity(oracle, dev, shape, causal, tile):
     from kernelcodegen_amd import ops
     B, H, S, D = shape
+    br, bc = tile
     Q, K, V = (inputs.normal(shape, 201, i) for i in range(3))
     for scale in (D ** -0.5, 1.0 / 3):
         ref = oracle.fmha(Q, K, V, scale=scale, causal=causal, stable=True)
         O = ops.fmha(_gpu(Q, dev), _gpu(K, dev), _gpu(V, dev), scale=scale, causal=causal,
-                     sched=dict(br=128, bc=bc)).cpu().numpy()
+                     sched=dict(br=br, bc=bc)).cpu().numpy()
         assert max(rel_err(O, ref)) < TOL_F32
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_f32_rising_row_maximum(oracle, dev, causal):
+    """Logits that climb along the key axis: by a few units per tile for some rows (the
+    reference maximum of the online softmax stays behind the true one) and by far more
+    than the rescale threshold for others (it is raised again and again), plus rows whose
+    largest logit comes first."""
+    from kernelcodegen_amd import ops
+    B, H, S, D = 1, 2, 384, 64
+    rng = np.random.default_rng(77)
+    K = rng.standard_normal((B, H, S, D)).astype(np.float32)
+    V = rng.standard_normal((B, H, S, D)).astype(np.float32)
+    Q = rng.standard_normal((B, H, S, D)).astype(np.float32) * np.float32(0.1)
+    ramp = np.linspace(0.0, 1.0, S, dtype=np.float32)
+    K[..., 0] = 60.0 * ramp          # logit contribution q0 * k0 * scale
+    Q[:, :, 0::3, 0] = 1.0           # climbs by ~60 over the sweep: repeated rescales
+    Q[:, :, 1::3, 0] = 0.05          # climbs by ~3: never exceeds the threshold after tile 0
+    Q[:, :, 2::3, 0] = -1.0          # falls: the first tile holds the maximum
+    ref = oracle.fmha(Q, K, V, scale=1.0, causal=causal, stable=True)
+    for tile in ((128, 32), (128, 64), (256, 32)):
+        O = ops.fmha(_gpu(Q, dev), _gpu(K, dev), _gpu(V, dev), scale=1.0, causal=causal,
+                     sched=dict(br=tile[0], bc=tile[1])).cpu().numpy()
+        assert max(rel_err(O, ref)) < TOL_F32, tile
 
 
 def test_f32_reference_graph_scale_one(oracle, dev):
