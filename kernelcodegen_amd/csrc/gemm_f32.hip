@@ -591,15 +591,23 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
     struct Cand {
       int bm, bn, bk, wm, wn;
       double eff;
+      double max_tiles;  // small tiles re-read A and B too often once the problem outgrows the L2s
     };
-    const Cand cands[] = {{256, 128, 16, 64, 64, 0.88}, {128, 128, 16, 64, 64, 0.86}, {64, 64, 32, 32, 32, 0.77}};
+    // efficiencies measured on problems that fill the chip evenly (fraction of MFMA peak)
+    const Cand cands[] = {{256, 128, 16, 64, 64, 0.91, 1e30},
+                          {128, 128, 16, 64, 64, 0.885, 1e30},
+                          {128, 64, 32, 64, 32, 0.85, 4096},
+                          {64, 64, 32, 32, 32, 0.84, 6400}};
     double best = -1.0;
     for (const Cand &c : cands) {
       const double tiles = static_cast<double>((M + c.bm - 1) / c.bm) * static_cast<double>((N + c.bn - 1) / c.bn);
+      if (tiles > c.max_tiles) continue;
       const double per_cu = static_cast<double>((static_cast<int64_t>(tiles) + kNumCu - 1) / kNumCu);
       // padding waste of ragged edges counts against a large tile too
       const double useful = (static_cast<double>(M) * N) / (tiles * c.bm * c.bn);
-      const double score = c.eff * useful * tiles / (per_cu * kNumCu);
+      // a CU left with a single 4-wave workgroup has one wave per SIMD to hide latency with
+      const double lonely = (c.bm * c.bn <= 128 * 128 && tiles <= kNumCu) ? 0.95 : 1.0;
+      const double score = c.eff * lonely * useful * tiles / (per_cu * kNumCu);
       if (score > best) {
         best = score;
         d = {c.bm, c.bn, c.bk, 8, c.wm, c.wn, 4, 64};
@@ -628,6 +636,7 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
   KCG_TRY(256, 128, 16, 4, 2, 2)
   KCG_TRY(256, 128, 32, 4, 2, 1)
   KCG_TRY(64, 64, 32, 2, 2, 2)
+  KCG_TRY(128, 64, 32, 2, 2, 2)
 #undef KCG_TRY
   return KCG_ERR_BAD_SCHEDULE;
 }

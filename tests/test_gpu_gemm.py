@@ -22,6 +22,7 @@ SCHEDS = [
     dict(block_m=128, block_n=128, block_k=32, wave_m=64, wave_n=64),
     dict(block_m=256, block_n=128, block_k=32, wave_m=64, wave_n=64),
     dict(block_m=64, block_n=64, block_k=32, wave_m=32, wave_n=32),
+    dict(block_m=128, block_n=64, block_k=32, wave_m=64, wave_n=32),
 ]
 
 
@@ -47,7 +48,7 @@ def test_tile_aligned_shapes(oracle, dev, shape, sched):
 
 @pytest.mark.parametrize("shape", [(1, 1, 1), (5, 3, 2), (131, 77, 19), (200, 136, 52), (129, 257, 33),
                                    (300, 128, 7), (64, 1000, 130)])
-@pytest.mark.parametrize("sched", [None, SCHEDS[1], SCHEDS[5]])
+@pytest.mark.parametrize("sched", [None, SCHEDS[1], SCHEDS[5], SCHEDS[6]])
 def test_ragged_shapes(oracle, dev, shape, sched):
     from kernelcodegen_amd import ops
     M, N, K = shape
