@@ -29,7 +29,7 @@ DIMS = [256, 512, 768, 1024, 1536, 2048, 3072, 4096, 5120, 6144, 7168, 8192, 921
 
 def _time(fn, iters):
     import torch
-    for _ in range(3):
+    for _ in range(max(3, iters // 4)):
         fn()
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
@@ -64,6 +64,13 @@ def main():
     dev = torch.device("cuda:0")
     shapes = [(4096, 2048, 1024)] + [(d, d, d) for d in DIMS if d <= args.max_dim]
     rows = []
+    # The shader clock takes some tens of milliseconds of load to settle: without this the
+    # first (small) shapes of the sweep are timed on a ramping clock.
+    W = torch.randn(4096, 4096, device=dev)
+    for _ in range(200):
+        ops.matmul(W, W, relu=args.relu)
+    torch.cuda.synchronize()
+    del W
     for (M, N, K) in shapes:
         A = torch.randn(M, K, device=dev)
         B = torch.randn(K, N, device=dev)
