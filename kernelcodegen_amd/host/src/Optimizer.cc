@@ -1,5 +1,7 @@
 #include "Optimizer/Optimizer.h"
 
+#include <limits>
+
 #include <algorithm>
 
 #include <cstdio>
@@ -429,6 +431,153 @@ bool FMHAOptimizer::applicable(ModuleOp &module) {
   return !call2callsMap.empty();
 }
 
+// The body of the fused function as an executable loop nest (the reference's design,
+// src/Optimizer/Optimizer.cc:948-1077 and 1191-1331: Br query rows per block, K/V swept in
+// Bc-row tiles, running maximum / sum / rescale), one query row per thread:
+//
+//   m = -inf; l = 0; acc[0..Hd) = 0
+//   for each K/V tile j:
+//     s[c]  = scale * sum_d Q[row, d] * K[j*Bc + c, d]          for the valid keys of the tile
+//     m'    = max(m, max_c s[c]);  alpha = exp(m - m')
+//     l     = l * alpha;  acc[d] = acc[d] * alpha;  m = m'
+//     p     = exp(s[c] - m);  l = l + p;  acc[d] = p * V[j*Bc + c, d] + acc[d]
+//   O[row, d] = acc[d] / l
+//
+// A key is valid when it is below the sequence length and, with the causal mask, not
+// beyond the query row; every valid row sees key 0 in tile 0, so m is finite from then on.
+// The nest is what the interpreter runs to check the fusion against the un-fused graph;
+// the GPU kernels implement the same recurrence on MFMA tiles.
+static void buildOnlineSoftmaxNest(Op *gridLevel, Op *blockLevel, Value Q, Value K, Value V, Value O,
+                                   int seqLen, int Hd, int Br, int Bc, float scale, bool causal) {
+  const DType f32 = DType::f32;
+  Value sBuf = Rewriter::alloc_buffer(OpHandle(blockLevel), MemorySpace::local, {Bc}, f32);
+  Value acc = Rewriter::alloc_buffer(OpHandle(blockLevel), MemorySpace::local, {Hd}, f32);
+  Value mNew = Rewriter::alloc_buffer(OpHandle(blockLevel), MemorySpace::local, {1}, f32);
+  Value ml = Rewriter::alloc_buffer(OpHandle(blockLevel), MemorySpace::local, {2}, f32);  // m, l
+  const int nGrid = static_cast<int>(gridLevel->args.size());
+  std::vector<LinExpr> batchIdx;
+  for (int i = 0; i + 1 < nGrid; ++i) batchIdx.emplace_back(gridLevel->arg(i));
+  Value qb = gridLevel->arg(nGrid - 1), t = blockLevel->arg(0);
+  LinExpr row;  // qb * Br + t
+  row.add(qb, Br).add(t, 1);
+  auto at = [&](const LinExpr &r, const LinExpr &c) {
+    auto idx = batchIdx;
+    idx.push_back(r);
+    idx.push_back(c);
+    return idx;
+  };
+  // this thread owns a row: t < Br and row < seqLen
+  LinExpr tInBlock(static_cast<int64_t>(Br - 1));
+  tInBlock.add(t, -1);
+  LinExpr rowInSeq(static_cast<int64_t>(seqLen - 1));
+  rowInSeq.add(row, -1);
+  Op *own = blockLevel->pushBack(makeIf({tInBlock, rowInSeq}));
+
+  Value zero = own->pushBack(makeConstant(0.0, f32))->result();
+  Value negInf = own->pushBack(makeConstant(-std::numeric_limits<double>::infinity(), f32))->result();
+  Value minusOne = own->pushBack(makeConstant(-1.0, f32))->result();
+  Value scaleV = own->pushBack(makeConstant(static_cast<double>(scale), f32))->result();
+  own->pushBack(makeStore(negInf, ml, {LinExpr(int64_t(0))}));
+  own->pushBack(makeStore(zero, ml, {LinExpr(int64_t(1))}));
+  {
+    Op *init = own->pushBack(makeFor(0, Hd, 1));
+    init->pushBack(makeStore(zero, acc, {LinExpr(init->arg(0))}));
+    init->pushBack(makeYield());
+  }
+  const int nTiles = (seqLen + Bc - 1) / Bc;
+  Op *tiles = own->pushBack(makeFor(0, nTiles, 1));
+  Value j = tiles->arg(0);
+  auto keyOf = [&](Value c) {
+    LinExpr key;
+    key.add(j, Bc).add(c, 1);
+    return key;
+  };
+  // `body(ifOp, c, key)` is emitted under the validity guard of key (j, c)
+  auto forValidKeys = [&](auto body) {
+    Op *loop = tiles->pushBack(makeFor(0, Bc, 1));
+    Value c = loop->arg(0);
+    LinExpr key = keyOf(c);
+    LinExpr inSeq(static_cast<int64_t>(seqLen - 1));
+    inSeq.add(key, -1);
+    std::vector<LinExpr> cons{inSeq};
+    if (causal) {
+      LinExpr notAfter = row;
+      notAfter.add(key, -1);
+      cons.push_back(notAfter);
+    }
+    Op *valid = loop->pushBack(makeIf(cons));
+    body(valid, c, key);
+    loop->pushBack(makeYield());
+  };
+  // s[c] = scale * <Q[row, :], K[key, :]>
+  forValidKeys([&](Op *g, Value c, const LinExpr &key) {
+    Op *dot = g->pushBack(makeFor(0, Hd, 1, {zero}));
+    Value q = dot->pushBack(makeLoad(Q, at(row, LinExpr(dot->arg(0)))))->result();
+    Value k = dot->pushBack(makeLoad(K, at(key, LinExpr(dot->arg(0)))))->result();
+    Value mul = dot->pushBack(makeBinary(OpKind::MulF, q, k))->result();
+    Value sum = dot->pushBack(makeBinary(OpKind::AddF, mul, dot->arg(1)))->result();
+    dot->pushBack(makeYield({sum}));
+    Value sc = g->pushBack(makeBinary(OpKind::MulF, dot->result(), scaleV))->result();
+    g->pushBack(makeStore(sc, sBuf, {LinExpr(c)}));
+  });
+  // m' = max(m, max_c s[c])
+  {
+    Value m = tiles->pushBack(makeLoad(ml, {LinExpr(int64_t(0))}))->result();
+    tiles->pushBack(makeStore(m, mNew, {LinExpr(int64_t(0))}));
+  }
+  forValidKeys([&](Op *g, Value c, const LinExpr &) {
+    Value cur = g->pushBack(makeLoad(mNew, {LinExpr(int64_t(0))}))->result();
+    Value sc = g->pushBack(makeLoad(sBuf, {LinExpr(c)}))->result();
+    Value mx = g->pushBack(makeBinary(OpKind::MaxF, cur, sc))->result();
+    g->pushBack(makeStore(mx, mNew, {LinExpr(int64_t(0))}));
+  });
+  // alpha = exp(m - m');  l *= alpha;  acc *= alpha;  m = m'
+  {
+    Value m = tiles->pushBack(makeLoad(ml, {LinExpr(int64_t(0))}))->result();
+    Value mn = tiles->pushBack(makeLoad(mNew, {LinExpr(int64_t(0))}))->result();
+    Value neg = tiles->pushBack(makeBinary(OpKind::MulF, mn, minusOne))->result();
+    Value diff = tiles->pushBack(makeBinary(OpKind::AddF, m, neg))->result();
+    Value alpha = tiles->pushBack(makeExp(diff))->result();
+    Value l = tiles->pushBack(makeLoad(ml, {LinExpr(int64_t(1))}))->result();
+    Value l2 = tiles->pushBack(makeBinary(OpKind::MulF, l, alpha))->result();
+    tiles->pushBack(makeStore(l2, ml, {LinExpr(int64_t(1))}));
+    Op *resc = tiles->pushBack(makeFor(0, Hd, 1));
+    Value a = resc->pushBack(makeLoad(acc, {LinExpr(resc->arg(0))}))->result();
+    Value a2 = resc->pushBack(makeBinary(OpKind::MulF, a, alpha))->result();
+    resc->pushBack(makeStore(a2, acc, {LinExpr(resc->arg(0))}));
+    resc->pushBack(makeYield());
+    tiles->pushBack(makeStore(mn, ml, {LinExpr(int64_t(0))}));
+  }
+  // p = exp(s[c] - m);  l += p;  acc[d] = p * V[key, d] + acc[d]
+  forValidKeys([&](Op *g, Value c, const LinExpr &key) {
+    Value m = g->pushBack(makeLoad(ml, {LinExpr(int64_t(0))}))->result();
+    Value neg = g->pushBack(makeBinary(OpKind::MulF, m, minusOne))->result();
+    Value sc = g->pushBack(makeLoad(sBuf, {LinExpr(c)}))->result();
+    Value diff = g->pushBack(makeBinary(OpKind::AddF, sc, neg))->result();
+    Value pv = g->pushBack(makeExp(diff))->result();
+    Value l = g->pushBack(makeLoad(ml, {LinExpr(int64_t(1))}))->result();
+    Value l2 = g->pushBack(makeBinary(OpKind::AddF, pv, l))->result();
+    g->pushBack(makeStore(l2, ml, {LinExpr(int64_t(1))}));
+    Op *upd = g->pushBack(makeFor(0, Hd, 1));
+    Value v = upd->pushBack(makeLoad(V, at(key, LinExpr(upd->arg(0)))))->result();
+    Value a = upd->pushBack(makeLoad(acc, {LinExpr(upd->arg(0))}))->result();
+    Value mul = upd->pushBack(makeBinary(OpKind::MulF, pv, v))->result();
+    Value a2 = upd->pushBack(makeBinary(OpKind::AddF, mul, a))->result();
+    upd->pushBack(makeStore(a2, acc, {LinExpr(upd->arg(0))}));
+    upd->pushBack(makeYield());
+  });
+  tiles->pushBack(makeYield());
+  // O[row, d] = acc[d] / l
+  {
+    Value l = own->pushBack(makeLoad(ml, {LinExpr(int64_t(1))}))->result();
+    Op *fin = own->pushBack(makeFor(0, Hd, 1));
+    Value a = fin->pushBack(makeLoad(acc, {LinExpr(fin->arg(0))}))->result();
+    Value o = fin->pushBack(makeBinary(OpKind::DivF, a, l))->result();
+    fin->pushBack(makeStore(o, O, at(row, LinExpr(fin->arg(0)))));
+    fin->pushBack(makeYield());
+  }
+}
+
 void FMHAOptimizer::applyOptimzer(ModuleOp &module) {
   auto cfg = [&](const char *key, int fallback) {
     auto it = fmhaConfig.find(key);
@@ -498,9 +647,16 @@ void FMHAOptimizer::applyOptimzer(ModuleOp &module) {
       const int padK = elem == DType::f32 ? 4 : 8, padV = elem == DType::f32 ? 8 : 32;
       Rewriter::alloc_buffer(OpHandle(gridLevel.op), MemorySpace::shared, {Bc, Hd + padV}, elem);
       Rewriter::alloc_buffer(OpHandle(gridLevel.op), MemorySpace::shared, {Bc, Hd + padK}, elem);
-      // per-lane registers: O^T accumulators (Hd/32 MFMA blocks x 16) and the running max / sum
-      Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {2}, DType::f32);
-      Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {Hd / 32 > 0 ? Hd / 32 : 1, 16}, DType::f32);
+      const bool detailed = cfg("SCHEDULE_DETAIL", 0) >= 1 && d1.batch.size() <= 2 && Br <= blockSize;
+      if (!detailed) {
+        // per-lane registers: O^T accumulators (Hd/32 MFMA blocks x 16) and the running max / sum
+        Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {2}, DType::f32);
+        Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {Hd / 32 > 0 ? Hd / 32 : 1, 16}, DType::f32);
+      } else {
+        buildOnlineSoftmaxNest(gridLevel.op, blockLevel.op, args[0], args[1], args[2], args[3], seq_len, Hd, Br, Bc,
+                               scale, causal);
+        funcOp.setAttr("kcg.schedule", "online_softmax");
+      }
       funcOp.setAttr("func.state", "gpu");
       funcOp.setAttr("kcg.Br", std::to_string(Br));
       funcOp.setAttr("kcg.Bc", std::to_string(Bc));

@@ -512,6 +512,119 @@ static void test_fmha_pattern_and_fusion() {
   CHECK(!again.applicable(graph.module));
 }
 
+// The fused function as an executable nest (SCHEDULE_DETAIL 1): online softmax over K/V
+// tiles, one query row per thread.  Run by the interpreter it must agree with the un-fused
+// three-operator graph (same inputs, literal softmax) and, with scale and the causal mask,
+// with a direct fp64 evaluation; sequence lengths that are no multiple of Br or Bc included.
+static void run_fused_attention_nest(int64_t b, int64_t h, int64_t s, int64_t d, int br, int bc, int threads,
+                                     float scale, bool causal, std::string *text) {
+  const size_t n = static_cast<size_t>(b * h * s * d);
+  std::vector<float> q(n), k(n), v(n);
+  unsigned seed = 4242u + static_cast<unsigned>(s) + (causal ? 7u : 0u);
+  auto rnd = [&]() {
+    seed = seed * 1664525u + 1013904223u;
+    return static_cast<float>(static_cast<int>(seed >> 8) % 2001 - 1000) / 1000.0f;
+  };
+  for (auto &x : q) x = rnd();
+  for (auto &x : k) x = rnd();
+  for (auto &x : v) x = rnd();
+  // direct evaluation in fp64
+  std::vector<double> expect(n);
+  for (int64_t bh = 0; bh < b * h; ++bh)
+    for (int64_t i = 0; i < s; ++i) {
+      std::vector<double> w(s, 0.0);
+      double sum = 0.0;
+      const int64_t last = causal ? i : s - 1;
+      for (int64_t j = 0; j <= last; ++j) {
+        double dot = 0.0;
+        for (int64_t c = 0; c < d; ++c) dot += double(q[(bh * s + i) * d + c]) * double(k[(bh * s + j) * d + c]);
+        w[j] = std::exp(dot * double(scale));
+        sum += w[j];
+      }
+      for (int64_t c = 0; c < d; ++c) {
+        double o = 0.0;
+        for (int64_t j = 0; j <= last; ++j) o += w[j] * double(v[(bh * s + j) * d + c]);
+        expect[(bh * s + i) * d + c] = o / sum;
+      }
+    }
+  KernelCodeGenerator gen;
+  gen.setLogMode(Log::Release);
+  auto &graph = gen.createGraph("fused_nest");
+  std::vector<int64_t> shape{b, h, s, d};
+  auto Q = graph.create<PlaceHolder>(shape, std::string{"float32"});
+  auto K = graph.create<PlaceHolder>(shape, std::string{"float32"});
+  auto V = graph.create<PlaceHolder>(shape, std::string{"float32"});
+  auto S = graph.create<BatchedMatmul>(Q, Layout::rowMajor, K, Layout::colMajor);
+  auto P = graph.create<Softmax>(S, -1, MemorySpace::inplace);
+  auto Ou = graph.create<BatchedMatmul>(P, Layout::rowMajor, V, Layout::rowMajor);
+  std::vector<float> unfused;
+  if (!causal && scale == 1.0f) {   // the reference graph itself has neither scale nor mask
+    Interpreter plain(graph.module);
+    plain.bind(Q, q.data());
+    plain.bind(K, k.data());
+    plain.bind(V, v.data());
+    CHECK(plain.run().empty());
+    const float *o = plain.buffer(Ou);
+    CHECK(o != nullptr);
+    if (o) unfused.assign(o, o + n);
+  }
+  gen.fmhaConfigs = {{{"BLOCK_SIZE", threads}, {"Br", br}, {"Bc", bc}, {"SCHEDULE_DETAIL", 1}}};
+  FMHAOptimizer::scale = scale;
+  FMHAOptimizer::causal = causal;
+  auto module = gen.optimize(graph);
+  FMHAOptimizer::scale = 1.0f;
+  FMHAOptimizer::causal = false;
+  const std::string problem = verify(module.get());
+  CHECK(problem.empty());
+  if (!problem.empty()) std::fprintf(stderr, "    verify: %s\n", problem.c_str());
+  auto fused = Analyzer::collectFunctions(module, "Fused_Multi_Head_Attention");
+  CHECK(fused.size() == 1 && fused[0].getAttr("kcg.schedule") == "online_softmax");
+  if (text) *text = module.str();
+  auto calls = Analyzer::collectFuncCalls(module);
+  CHECK(calls.size() == 1);
+  if (calls.size() != 1) return;
+  std::vector<float> o(n, -7.0f);
+  Interpreter interp(module);   // optimize() works on a copy of the graph's module: bind the copy's buffers
+  auto operands = calls[0].getArgOperands();
+  interp.bind(operands[0], q.data());
+  interp.bind(operands[1], k.data());
+  interp.bind(operands[2], v.data());
+  interp.bind(operands[3], o.data());
+  const std::string err = interp.run();
+  CHECK(err.empty());
+  if (!err.empty()) std::fprintf(stderr, "    interpreter: %s\n", err.c_str());
+  double worst = 0.0, worstUnfused = 0.0;
+  for (size_t i = 0; i < n; ++i) {
+    worst = std::max(worst, std::fabs(double(o[i]) - expect[i]));
+    if (!unfused.empty()) worstUnfused = std::max(worstUnfused, std::fabs(double(o[i]) - double(unfused[i])));
+  }
+  if (worst >= 2e-6) std::fprintf(stderr, "    worst %g, against the un-fused graph %g\n", worst, worstUnfused);
+  CHECK(worst < 2e-6);          // |O| <= max|V| = 1
+  CHECK(worstUnfused < 2e-6);
+  // the fused module still binds to the kernel library from its attributes
+  if (d == 64 || d == 128) {
+    auto bindings = gen.bind(module);
+    CHECK(bindings.size() == 1 && bindings[0].kind == KernelBinding::Fmha);
+  }
+}
+
+static void test_fused_attention_nest() {
+  std::string text;
+  run_fused_attention_nest(1, 2, 40, 32, 16, 8, 32, 1.0f, false, &text);   // 2.5 query blocks, 5 tiles
+  CHECK(contains(text, "kcg.schedule = \"online_softmax\""));
+  CHECK(count(text, "math.exp") == 2);                 // rescale factor and P
+  CHECK(count(text, "arith.maxf") == 1 && count(text, "arith.divf") == 1);
+  CHECK(contains(text, "memref<8xf32, 3>") && contains(text, "memref<32xf32, 3>"));   // S tile, O row
+  CHECK(contains(text, "affine.if affine_set<(d0, d1) : (-d0 + 15 >= 0, d1 * -16 - d0 + 39 >= 0)>"));
+  CHECK(!contains(text, "func.func @Softmax") && !contains(text, "func.func @BatchMatmul"));
+  run_fused_attention_nest(2, 1, 33, 16, 16, 16, 16, 0.25f, true, &text);   // ragged, causal, scaled
+  CHECK(count(text, "affine.if") == 4);                // row guard + three key-validity guards
+  // key < S and key <= row, with key = tile * 16 + c and row = block * 16 + thread
+  CHECK(count(text, "(d0 * -16 - d1 + 32 >= 0, d2 * 16 + d3 + d0 * -16 - d1 >= 0)") == 3);
+  run_fused_attention_nest(1, 1, 128, 64, 128, 32, 256, 0.125f, true, nullptr);   // the kernel's own tile, bindable
+  run_fused_attention_nest(1, 1, 9, 8, 4, 4, 4, 1.0f, false, nullptr);
+}
+
 static void test_fmha_pattern_rejections() {
   {  // softmax result used twice: not fusable
     KernelCodeGenerator gen;
@@ -781,6 +894,7 @@ int main() {
       {"relu_softmax_batched_matmul_semantics", test_relu_softmax_batched_matmul_semantics},
       {"batched_matmul_layouts", test_batched_matmul_layouts},
       {"fmha_pattern_and_fusion", test_fmha_pattern_and_fusion},
+      {"fused_attention_nest", test_fused_attention_nest},
       {"fmha_pattern_rejections", test_fmha_pattern_rejections},
       {"facade_matmul_demo", test_facade_matmul_demo},
       {"facade_config_search_and_reference_tile", test_facade_config_search_and_reference_tile},
