@@ -27,6 +27,17 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 TRAFFIC_BYTES = {"gemm_cfg1": 771442602, "fmha_cfg3": 134328811, "fmha_cfg4": 795121940}
 
 
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def time_launches(fn, steps, warmup):
     """(wall ms per step, HIP-event ms per launch) over `steps` launches of fn."""
     import torch
@@ -119,6 +130,7 @@ def main():
         rms = float(np.sqrt((ref.astype(np.float64) ** 2).mean()))
         out["cpu_baseline"] = {
             "value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.num_threads(),
+            "cpu_model": _cpu_model(),
             "kind": "port", "sample": "the whole configs[1] workload (4096^3 matmul + ReLU), best of "
                                       "3 runs, %.2f s wall each" % dt,
             "gpu_vs_cpu_max_rel_err": float((d / np.maximum(np.abs(ref), rms)).max()),
