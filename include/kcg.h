@@ -104,8 +104,9 @@ KCG_API int kcg_gemm_f32_query(int64_t M, int64_t N, int64_t K,
  * 38-41; Br = HdxBr / Hd, Bc = BrxBc / Br, src/Optimizer/Optimizer.cc:1136-1144)
  * reduced to the two tile extents.  NULL or 0 selects the gfx950 default. */
 typedef struct kcg_fmha_sched {
-  int32_t br; /* query rows per workgroup                                      */
-  int32_t bc; /* key/value rows per inner step                                 */
+  int32_t br; /* query rows per workgroup: 128 (4 waves) or 256 (8 waves)      */
+  int32_t bc; /* key/value rows per inner step: fp32 32 or 64 (not 256 x 64 at
+               * D = 128), bf16 64                                             */
 } kcg_fmha_sched;
 
 /* O = softmax(scale * Q.K^T [+ causal mask]) . V, all [B,H,S,D] contiguous fp32.
