@@ -76,3 +76,32 @@ def test_unfused_graph_matches_fused_kernel(oracle, dev):
     assert max(rel_err(O3, ref)) < 1e-4
     Of = ops.fmha(dQ, dK, dV, scale=1.0, causal=False).cpu().numpy()
     assert max(rel_err(Of, O3)) < 1e-4
+
+
+def test_launches_follow_the_callers_stream(oracle, dev):
+    """Every entry point is asynchronous on the stream it is given: work queued on a side
+    stream (default priority) is ordered after what that stream already holds and is not
+    visible to the host before the stream is synchronised; two streams run independently."""
+    import torch
+    from kernelcodegen_amd import ops
+    M = N = K = 512
+    A = inputs.normal((M, K), 77, 0)
+    B = inputs.normal((K, N), 77, 1)
+    ref = oracle.relu(oracle.matmul(A, B))
+    tA, tB = _gpu(A, dev), _gpu(B, dev)
+    side, other = torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        # the producer of the operand and its consumer are both queued on `side`
+        tA2 = tA * 2.0
+        C = ops.matmul(tA2, tB, relu=True)
+        D = ops.relu(C * -1.0)
+    with torch.cuda.stream(other):
+        shape = (1, 2, 256, 64)
+        Q, Kk, V = (inputs.normal(shape, 78, i) for i in range(3))
+        O = ops.fmha(_gpu(Q, dev), _gpu(Kk, dev), _gpu(V, dev), scale=0.125, causal=True)
+    side.synchronize()
+    other.synchronize()
+    assert max(rel_err(C.cpu().numpy(), 2.0 * ref)) < 1e-4
+    assert float(D.abs().max()) == 0.0          # relu(-relu(x)) == 0
+    assert max(rel_err(O.cpu().numpy(), oracle.fmha(Q, Kk, V, scale=0.125, causal=True, stable=True))) < 1e-4
