@@ -105,3 +105,46 @@ def test_launches_follow_the_callers_stream(oracle, dev):
     assert max(rel_err(C.cpu().numpy(), 2.0 * ref)) < 1e-4
     assert float(D.abs().max()) == 0.0          # relu(-relu(x)) == 0
     assert max(rel_err(O.cpu().numpy(), oracle.fmha(Q, Kk, V, scale=0.125, causal=True, stable=True))) < 1e-4
+
+
+def test_entry_points_can_be_captured_in_a_graph(dev):
+    """The entry points neither allocate nor synchronise, so a caller may record them into a
+    HIP graph.  The graph is replayed several times with eager work and synchronisations in
+    between and new operand contents each time; every replay must equal the eager result."""
+    import torch
+    from kernelcodegen_amd import ops
+    torch.manual_seed(5)
+    A = torch.randn(384, 256, device=dev)
+    B = torch.randn(256, 512, device=dev)
+    C = torch.empty(384, 512, device=dev)
+    Q = torch.randn(1, 2, 320, 128, device=dev)
+    K = torch.randn_like(Q)
+    V = torch.randn_like(Q)
+    O = torch.empty_like(Q)
+    Qb, Kb, Vb = Q.bfloat16(), K.bfloat16(), V.bfloat16()
+    Ob = torch.empty_like(Qb)
+
+    def launch_all():
+        ops.matmul(A, B, relu=True, out=C)
+        ops.fmha(Q, K, V, scale=0.09, causal=True, out=O)
+        ops.fmha(Qb, Kb, Vb, scale=0.09, causal=True, out=Ob)
+
+    launch_all()                      # first use of each kernel outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch_all()
+    for rep in range(3):
+        A.normal_()
+        Q.normal_()
+        Qb.copy_(Q)
+        launch_all()
+        torch.cuda.synchronize()
+        want = (C.clone(), O.clone(), Ob.clone())
+        C.fill_(-1.0)
+        O.fill_(-1.0)
+        Ob.fill_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(C, want[0]) and torch.equal(O, want[1]) and torch.equal(Ob, want[2]), rep
