@@ -148,3 +148,40 @@ def test_entry_points_can_be_captured_in_a_graph(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(C, want[0]) and torch.equal(O, want[1]) and torch.equal(Ob, want[2]), rep
+
+
+def test_concurrent_host_threads(oracle, dev):
+    """The library keeps no state between calls: four host threads launch different
+    problems on their own streams at the same time (ctypes releases the GIL around the
+    call) and each gets its own correct result."""
+    import threading
+    import torch
+    from kernelcodegen_amd import ops
+    shapes = [(256, 128, 96), (130, 70, 33), (512, 256, 64), (64, 64, 512)]
+    hostA = [inputs.normal((m, k), 300 + i, 0) for i, (m, n, k) in enumerate(shapes)]
+    hostB = [inputs.normal((k, n), 300 + i, 1) for i, (m, n, k) in enumerate(shapes)]
+    devA = [_gpu(a, dev) for a in hostA]
+    devB = [_gpu(b, dev) for b in hostB]
+    torch.cuda.synchronize()
+    results, errors = [None] * len(shapes), []
+
+    def work(i):
+        try:
+            stream = torch.cuda.Stream(device=dev)
+            with torch.cuda.stream(stream):
+                out = None
+                for _ in range(20):
+                    out = ops.matmul(devA[i], devB[i], relu=True)
+            stream.synchronize()
+            results[i] = out.cpu().numpy()
+        except Exception as e:      # surfaced in the main thread below
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(shapes))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(len(shapes)):
+        assert max(rel_err(results[i], oracle.relu(oracle.matmul(hostA[i], hostB[i])))) < 1e-4, shapes[i]
