@@ -277,6 +277,26 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 #define KCG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define KCG_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
+// One wave-wide direct load: lane l's 16 bytes at (uniform base + off) go to LDS byte
+// address lds_addr + 16 * l.  Issued from assembly so that the address is formed by the
+// instruction itself (scalar base + 32-bit lane offset); the intrinsic materialises a
+// 64-bit address per lane with VALU work, which on this chip comes out of fp32 MFMA time.
+// M0 (the LDS base of the load) is saved and restored around the instruction.
+__device__ __forceinline__ void direct_load_16B(const void *base, unsigned off, unsigned lds_addr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  unsigned saved_m0;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %2, %3\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0)
+      : "s"(lds_addr), "v"(off), "s"(base)
+      : "memory");
+#endif
+}
+
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 struct GemmDlTile {
   static constexpr int kWaves = WAVES_M * WAVES_N;
@@ -346,6 +366,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // ---- direct loads: uniform slice base + per-lane 32-bit byte offsets ----
+  const int lds_base = static_cast<int>(reinterpret_cast<uintptr_t>(lds));  // LDS byte address
   unsigned oa[T::kInstrA];
   unsigned ob[T::kInstrB];
 #pragma unroll
@@ -367,12 +388,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   // load l of the slice at (ga, gb) into the stage at float offset stage_off
   auto issue_one = [&](int stage_off, int l) {
     if (l < T::kInstrA) {
-      float *sa = lds + stage_off + (wave * T::kInstrA + l) * 256;
-      __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(ga + oa[l]), KCG_LDS_PTR(sa), 16, 0, 0);
+      const int sa = lds_base + (stage_off + (wave * T::kInstrA + l) * 256) * 4;
+      direct_load_16B(ga, oa[l], static_cast<unsigned>(sa));
     } else {
       const int i = l - T::kInstrA;
-      float *sb = lds + stage_off + T::kFloatsA + (wave * T::kInstrB + i) * T::kRunB;
-      __builtin_amdgcn_global_load_lds(KCG_GLOBAL_PTR(gb + ob[i]), KCG_LDS_PTR(sb), 16, 0, 0);
+      const int sb = lds_base + (stage_off + T::kFloatsA + (wave * T::kInstrB + i) * T::kRunB) * 4;
+      direct_load_16B(gb, ob[i], static_cast<unsigned>(sb));
     }
   };
   // The loop body is kept free of branches (after a join the compiler's wait-count
@@ -425,7 +446,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   auto next_stage = [](int off) {
     return off == (T::kStages - 1) * T::kStageFloats ? 0 : off + T::kStageFloats;
   };
-  const int lds_base = static_cast<int>(reinterpret_cast<uintptr_t>(lds));
 
   // Publishes the slice requested before the newest one: the wave waits for its
   // own loads of that slice and for its LDS reads, then joins the barrier.  A bare
