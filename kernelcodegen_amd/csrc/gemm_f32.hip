@@ -26,6 +26,8 @@
 // read of A) and the j-th MFMA of the group consumes k = 4h + j from both
 // operands.  The set of products summed into each C element is unchanged; only
 // their order differs from the ascending-k order of the reference nest.
+#include <type_traits>
+
 #include "kcg_common.h"
 
 namespace kcg {
@@ -411,19 +413,26 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   // every MFMA group, which undoes the operand prefetch.  The reads are therefore
   // issued from inline assembly, invisible to that bookkeeping, and waited for by
   // hand: LDS reads return in order, so "all but the newest n" is lgkmcnt(n).
-  int a_off[BK / 8];  // byte offsets inside a stage, swizzle folded in
+  // Per-lane LDS byte addresses, one set per stage (swizzle folded in): the slice loop is
+  // unrolled over the three stages so that no address arithmetic is left in it -- on this
+  // chip every VALU instruction between fp32 MFMAs is paid for in matrix time.
+  int a_addr[T::kStages][BK / 8];
+  int b_addr[T::kStages];
 #pragma unroll
-  for (int kk = 0; kk < BK / 8; ++kk)
-    a_off[kk] = ((wm * T::kWaveM + r32) * BK + 4 * ((2 * kk) ^ half ^ T::fa(r32))) * 4;
-  const int b_off = (T::kFloatsA + half * T::brow(4) + wn * T::kWaveN + r32) * 4;
+  for (int st = 0; st < T::kStages; ++st) {
+#pragma unroll
+    for (int kk = 0; kk < BK / 8; ++kk)
+      a_addr[st][kk] = lds_base + (st * T::kStageFloats + (wm * T::kWaveM + r32) * BK +
+                                   4 * ((2 * kk) ^ half ^ T::fa(r32))) * 4;
+    b_addr[st] = lds_base + (st * T::kStageFloats + T::kFloatsA + half * T::brow(4) + wn * T::kWaveN + r32) * 4;
+  }
 
   float4_t fa[2][T::kTilesM];
   float fb[2][T::kTilesN];
   float4_t na[T::kTilesM];
   float nb[T::kTilesN];
-  // stage_addr: LDS byte address of the stage
-  auto read_a = [&](int stage_addr, int kk, float4_t(&dst)[T::kTilesM]) {
-    const int addr = stage_addr + a_off[kk];
+  auto read_a = [&](int stage, int kk, float4_t(&dst)[T::kTilesM]) {
+    const int addr = a_addr[stage][kk];
 #pragma unroll
     for (int i = 0; i < T::kTilesM; ++i)
       asm volatile("ds_read_b128 %0, %1 offset:%2"
@@ -431,8 +440,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
                    : "v"(addr), "n"(i * 32 * BK * 4)
                    : "memory");
   };
-  auto read_b = [&](int stage_addr, int s, float(&dst)[T::kTilesN]) {
-    const int addr = stage_addr + b_off;
+  auto read_b = [&](int stage, int s, float(&dst)[T::kTilesN]) {
+    const int addr = b_addr[stage];
 #pragma unroll
     for (int n = 0; n < T::kTilesN; ++n)
       asm volatile("ds_read_b32 %0, %1 offset:%2"
@@ -443,9 +452,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   constexpr int kReadsA = T::kTilesM;  // LDS instructions per read_a / read_b
   constexpr int kReadsB = T::kTilesN;
   static_assert((T::brow(BK - 1) + BN) * 4 < 65536 && BM * BK * 4 < 65536, "ds_read offset field");
-  auto next_stage = [](int off) {
-    return off == (T::kStages - 1) * T::kStageFloats ? 0 : off + T::kStageFloats;
-  };
 
   // Publishes the slice requested before the newest one: the wave waits for its
   // own loads of that slice and for its LDS reads, then joins the barrier.  A bare
@@ -462,22 +468,48 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   };
 
   const int ktiles = K / BK;
+  // The slice loop runs whole groups of three slices (stages 0, 1, 2); the ktiles % 3
+  // slices in front of the first group use the last stages of the ring, so that the
+  // first group starts at stage 0.
+  const int peeled = ktiles % 3;
+  const int first_stage = (3 - peeled) % 3;
+  const int second_stage = (first_stage + 1) % 3;
 #pragma unroll
-  for (int l = 0; l < kLoadsPerSlice; ++l) issue_one(0, l);
+  for (int l = 0; l < kLoadsPerSlice; ++l) issue_one(first_stage * T::kStageFloats, l);
   advance_if(ktiles > 1);
 #pragma unroll
-  for (int l = 0; l < kLoadsPerSlice; ++l) issue_one(T::kStageFloats, l);
+  for (int l = 0; l < kLoadsPerSlice; ++l) issue_one(second_stage * T::kStageFloats, l);
   advance_if(ktiles > 2);
   publish();
-  read_a(lds_base, 0, na);
-  read_b(lds_base, 0, nb);
+  // Outstanding LDS reads must not cross a control-flow join: the compiler may copy their
+  // destination registers there, before the data has arrived.
+  auto drain_reads = [&]() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < T::kTilesM; ++i) asm volatile("" : "+v"(na[i]));
+#pragma unroll
+    for (int n = 0; n < T::kTilesN; ++n) asm volatile("" : "+v"(nb[n]));
+  };
+  if (first_stage == 0) {
+    read_a(0, 0, na);
+    read_b(0, 0, nb);
+    drain_reads();
+  } else if (first_stage == 1) {
+    read_a(1, 0, na);
+    read_b(1, 0, nb);
+    drain_reads();
+  } else {
+    read_a(2, 0, na);
+    read_b(2, 0, nb);
+    drain_reads();
+  }
 
-  int st = 0;  // stage (float offset) holding slice kt
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const int st1 = next_stage(st);
-    const int st2 = next_stage(st1);
-    const int st_addr = lds_base + st * 4;
-    const int st1_addr = lds_base + st1 * 4;
+  // One K slice held in stage ST (a compile-time constant: all LDS addresses and the
+  // direct-load targets are immediates or loop-invariant registers).
+  auto slice = [&](auto stage_c, int kt) {
+    constexpr int ST = decltype(stage_c)::value;
+    constexpr int ST1 = (ST + 1) % T::kStages;
+    constexpr int ST2 = (ST + 2) % T::kStages;
     // the reads of step 0, issued after the previous barrier, are the newest in flight
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
@@ -490,18 +522,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       // burst by every wave of the CU queue up at the address unit.
 #pragma unroll
       for (int l = 0; l < kLoadsPerSlice; ++l)
-        if (s == 1 + l * (T::kSteps - 2) / kLoadsPerSlice) issue_one(st2, l);
+        if (s == 1 + l * (T::kSteps - 2) / kLoadsPerSlice) issue_one(ST2 * T::kStageFloats, l);
       if (s + 1 < T::kSteps) {
         const bool with_a = (s + 1) % 4 == 0;
-        if (with_a) read_a(st_addr, (s + 1) / 4, fa[((s + 1) / 4) & 1]);
-        read_b(st_addr, s + 1, fb[(s + 1) & 1]);
+        if (with_a) read_a(ST, (s + 1) / 4, fa[((s + 1) / 4) & 1]);
+        read_b(ST, s + 1, fb[(s + 1) & 1]);
         // operands of step s were requested one step ago: all but this step's reads
         if (with_a) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsA + kReadsB) : "memory");
         else asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsB) : "memory");
       } else {
         publish();  // includes lgkmcnt(0): the operands of the last step are in
-        read_a(st1_addr, 0, na);
-        read_b(st1_addr, 0, nb);
+        read_a(ST1, 0, na);
+        read_b(ST1, 0, nb);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -513,7 +545,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       __builtin_amdgcn_sched_barrier(0);
     }
     advance_if(kt + 3 < ktiles);
-    st = st1;
+  };
+  static_assert(T::kStages == 3, "the slice loop is unrolled over three stages");
+  if (peeled == 2) {
+    slice(std::integral_constant<int, 1>{}, 0);
+    drain_reads();
+  }
+  if (peeled >= 1) {
+    slice(std::integral_constant<int, 2>{}, peeled - 1);
+    drain_reads();
+  }
+  for (int kt = peeled; kt < ktiles; kt += 3) {
+    slice(std::integral_constant<int, 0>{}, kt);
+    slice(std::integral_constant<int, 1>{}, kt + 1);
+    slice(std::integral_constant<int, 2>{}, kt + 2);
   }
   // LDS may be handed to another workgroup once this one retires: drain the loads.
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), lgkmcnt/expcnt untouched
