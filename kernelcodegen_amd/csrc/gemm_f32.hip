@@ -51,8 +51,19 @@ struct GemmTile {
   static_assert((BM * BK / 4) % kThreads == 0 && (BK * BN / 4) % kThreads == 0, "load split");
 };
 
+// Four consecutive floats from an address that is only known to be 4-byte aligned.
+__device__ __forceinline__ float4_t load4_dword_aligned(const float *p) {
+  struct __attribute__((packed, aligned(4))) Quad {
+    float v[4];
+  };
+  const Quad q = *reinterpret_cast<const Quad *>(p);
+  return float4_t{q.v[0], q.v[1], q.v[2], q.v[3]};
+}
+
 // FULL: M % BM == 0, N % BN == 0, K % BK == 0 and 16-byte aligned rows, so that
-// no bounds checks are needed and every global access is a dwordx4.
+// no bounds checks are needed and every global access is a dwordx4.  Otherwise
+// tiles inside C still take vector loads for all but the last, partial K slice.
+
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool FULL, int MIN_WAVES>
 __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
@@ -92,6 +103,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 
   float4_t ra[T::kLoadsA];
   float4_t rb[T::kLoadsB];
+  // ragged problems: a tile that lies wholly inside C needs bounds checks only in the
+  // last, partial K slice
+  const bool tile_inside = (m0 + BM <= M) && (n0 + BN <= N);
 
   // Transfer g of a K slice: g < kLoadsA moves one float4 of A per thread, the
   // rest one float4 of B.  load_one: global -> registers; store_one: registers -> LDS.
@@ -105,13 +119,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       const int gk = k0 + c4 * 4;
       if (FULL) {
         ra[g] = *reinterpret_cast<const float4_t *>(A + gr * K + gk);
+      } else if (tile_inside && k0 + BK <= K) {
+        // interior tile of a ragged problem: no element is out of range, but rows need
+        // not start on a 16-byte boundary
+        ra[g] = load4_dword_aligned(A + gr * K + gk);
       } else {
         float4_t v = {0.f, 0.f, 0.f, 0.f};
         if (gr < M) {
           const float *p = A + gr * K;
+          if (gk + 3 < K) {
+            v = load4_dword_aligned(p + gk);
+          } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (gk + e < K) v[e] = p[gk + e];
+            for (int e = 0; e < 4; ++e)
+              if (gk + e < K) v[e] = p[gk + e];
+          }
         }
         ra[g] = v;
       }
@@ -124,13 +146,19 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       const int gn = n0 + c4 * 4;
       if (FULL) {
         rb[i] = *reinterpret_cast<const float4_t *>(B + gk * N + gn);
+      } else if (tile_inside && k0 + BK <= K) {
+        rb[i] = load4_dword_aligned(B + gk * N + gn);
       } else {
         float4_t v = {0.f, 0.f, 0.f, 0.f};
         if (gk < K) {
           const float *p = B + gk * N;
+          if (gn + 3 < N) {
+            v = load4_dword_aligned(p + gn);
+          } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (gn + e < N) v[e] = p[gn + e];
+            for (int e = 0; e < 4; ++e)
+              if (gn + e < N) v[e] = p[gn + e];
+          }
         }
         rb[i] = v;
       }
