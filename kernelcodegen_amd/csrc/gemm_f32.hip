@@ -361,7 +361,14 @@ struct GemmDlTile {
   }
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, int MIN_WAVES>
+// RAGGED: M, N need not divide the tile and K need not divide BK (K and N are multiples of
+// 4 and K >= BK).  Rows of A at and beyond M and 16-byte column chunks of B at and beyond N
+// only feed elements of C that are never stored, so their lanes simply fetch the last
+// valid row / chunk instead (a loop-invariant change of the lane offsets).  The last,
+// partial K slice is the one place that needs zeros: its direct loads re-fetch the last
+// full slice (never out of range) and the stage is then rewritten through registers, once
+// per tile.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool RAGGED, int MIN_WAVES>
 __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_dl_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
     int K, int tiles_m, int tiles_n, int group_m) {
@@ -404,12 +411,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
     const int idx = (wave * T::kInstrA + i) * 256 + lane * 4;  // float index in the LDS A tile
     const int row = idx / BK;
     const int c_log = ((idx % BK) / 4) ^ T::fa(row);
-    oa[i] = static_cast<unsigned>(row * K + 4 * c_log) * 4u;
+    const int grow = RAGGED ? (row < M - m0 ? row : M - m0 - 1) : row;
+    oa[i] = static_cast<unsigned>(grow * K + 4 * c_log) * 4u;
   }
 #pragma unroll
   for (int i = 0; i < T::kInstrB; ++i) {
     const int idx = (wave * T::kInstrB + i) * 256 + lane * 4;  // float index in the unpadded B tile
-    ob[i] = static_cast<unsigned>((idx / BN) * N + idx % BN) * 4u;
+    const int col = idx % BN;
+    const int gcol = RAGGED ? (col < N - n0 ? col : N - n0 - 4) : col;
+    ob[i] = static_cast<unsigned>((idx / BN) * N + gcol) * 4u;
   }
   const char *ga = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
   const char *gb = reinterpret_cast<const char *>(B + n0);
@@ -495,7 +505,35 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
     asm volatile("" ::: "memory");
   };
 
-  const int ktiles = K / BK;
+  const int kfull = K / BK;                      // slices the direct loads may fetch
+  const int ktiles = RAGGED ? (K + BK - 1) / BK : kfull;
+  // The last, partial slice (RAGGED): rewritten through registers with zeros beyond K.
+  // Lane L of load l owns the same 16 bytes of the stage as in the direct load.
+  auto rewrite_tail = [&](int stage_off) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stage's own direct loads have landed
+    const int k0 = kfull * BK;
+#pragma unroll
+    for (int l = 0; l < kLoadsPerSlice; ++l) {
+      float4_t v = {0.f, 0.f, 0.f, 0.f};
+      if (l < T::kInstrA) {
+        const int idx = (wave * T::kInstrA + l) * 256 + lane * 4;
+        const int row = idx / BK;
+        const int k = k0 + 4 * (((idx % BK) / 4) ^ T::fa(row));
+        const int grow = m0 + (row < M - m0 ? row : M - m0 - 1);
+        if (k < K) v = *reinterpret_cast<const float4_t *>(A + static_cast<int64_t>(grow) * K + k);
+        *reinterpret_cast<float4_t *>(lds + stage_off + idx) = v;
+      } else {
+        const int i = l - T::kInstrA;
+        const int idx = (wave * T::kInstrB + i) * 256 + lane * 4;
+        const int krow = k0 + idx / BN;
+        const int col = idx % BN;
+        const int gcol = n0 + (col < N - n0 ? col : N - n0 - 4);
+        if (krow < K) v = *reinterpret_cast<const float4_t *>(B + static_cast<int64_t>(krow) * N + gcol);
+        *reinterpret_cast<float4_t *>(lds + stage_off + T::kFloatsA + (wave * T::kInstrB + i) * T::kRunB +
+                                      lane * 4) = v;
+      }
+    }
+  };
   // The slice loop runs whole groups of three slices (stages 0, 1, 2); the ktiles % 3
   // slices in front of the first group use the last stages of the ring, so that the
   // first group starts at stage 0.
@@ -504,10 +542,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   const int second_stage = (first_stage + 1) % 3;
 #pragma unroll
   for (int l = 0; l < kLoadsPerSlice; ++l) issue_one(first_stage * T::kStageFloats, l);
-  advance_if(ktiles > 1);
+  advance_if(kfull > 1);
 #pragma unroll
   for (int l = 0; l < kLoadsPerSlice; ++l) issue_one(second_stage * T::kStageFloats, l);
-  advance_if(ktiles > 2);
+  advance_if(kfull > 2);
   publish();
   // Outstanding LDS reads must not cross a control-flow join: the compiler may copy their
   // destination registers there, before the data has arrived.
@@ -544,6 +582,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
     for (int i = 0; i < T::kTilesM; ++i) fa[0][i] = na[i];
 #pragma unroll
     for (int n = 0; n < T::kTilesN; ++n) fb[0][n] = nb[n];
+    // (no LDS read is outstanding here: a safe place for control flow)
+    if (RAGGED && kfull != ktiles && kt == ktiles - 2) rewrite_tail(ST1 * T::kStageFloats);
 #pragma unroll
     for (int s = 0; s < T::kSteps; ++s) {
       // The loads of slice kt+2 are spread over the steps: requests issued in one
@@ -572,7 +612,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
                                                            acc[i][n], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
-    advance_if(kt + 3 < ktiles);
+    advance_if(kt + 3 < kfull);
   };
   static_assert(T::kStages == 3, "the slice loop is unrolled over three stages");
   if (peeled == 2) {
@@ -601,7 +641,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
         const int row = m0 + wm * T::kWaveM + i * 32 + 8 * (e / 4) + 4 * half + (e % 4);
         float v = acc[i][n][e];
         if (RELU) v = relu_maxf(v);
-        C[static_cast<int64_t>(row) * N + col] = v;
+        if (!RAGGED || (row < M && col < N)) C[static_cast<int64_t>(row) * N + col] = v;
       }
     }
   }
@@ -616,6 +656,8 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
   if (tiles_m * tiles_n > 0x7fffffffLL || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL)
     return KCG_ERR_BAD_SHAPE;
   const bool full = (M % BM == 0) && (N % BN == 0) && (K % BK == 0) && aligned16(A) && aligned16(B);
+  // the direct-load kernel also takes ragged problems whose rows keep 16-byte alignment
+  const bool ragged_dl = !full && (K % 4 == 0) && (N % 4 == 0) && K >= BK && aligned16(A) && aligned16(B);
   const bool relu = epilogue == KCG_EPILOGUE_RELU;
   if (info) {
     info->grid[0] = static_cast<int>(tiles_m * tiles_n);
@@ -626,9 +668,9 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
     info->waves_per_block = WAVES_M * WAVES_N;
     const char *kind = "";
     if constexpr (BK == 16 || BK == 32) {
-      if (full) {  // the direct-load kernel takes full-tile problems
+      if ((full || ragged_dl) && K < (1 << 22) && N < (1 << 24)) {
         info->lds_bytes = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>::kLdsBytes;
-        kind = "_dl";
+        kind = full ? "_dl" : "_dl_ragged";
       }
     }
     snprintf(info->kernel, sizeof info->kernel, "gemm_f32_%dx%dx%d_w%dx%d%s", BM, BN, BK, WAVES_M,
@@ -640,15 +682,18 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
   if constexpr (BK == 16 || BK == 32) {
     using TD = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>;
     // the direct-load kernel addresses a slice with 32-bit byte offsets
-    if (full && K < (1 << 22) && N < (1 << 24)) {
+    if ((full || ragged_dl) && K < (1 << 22) && N < (1 << 24)) {
       auto launch_dl = [&](auto kern) {
         if (!allow_lds(kern, TD::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
         return launch(kern, grid, block, TD::kLdsBytes, stream, A, B, C, static_cast<int>(M),
                       static_cast<int>(N), static_cast<int>(K), static_cast<int>(tiles_m),
                       static_cast<int>(tiles_n), group_m);
       };
-      return relu ? launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, true, MIN_WAVES>)
-                  : launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, MIN_WAVES>);
+      if (full)
+        return relu ? launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, true, false, MIN_WAVES>)
+                    : launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, false, MIN_WAVES>);
+      return relu ? launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, true, true, MIN_WAVES>)
+                  : launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, true, MIN_WAVES>);
     }
   }
 #define KCG_LAUNCH(RELU_, FULL_)                                                                 \

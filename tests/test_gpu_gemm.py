@@ -59,6 +59,48 @@ def test_ragged_shapes(oracle, dev, shape, sched):
     assert max(rel_err(C, oracle.relu(oracle.matmul(A, B)))) < TOL
 
 
+# K and N multiples of 4, K at least one slice: the direct-load kernel takes these ragged
+# problems itself (rows and column chunks past the edge are clamped, the partial last K
+# slice is rewritten with zeros).  One slice only, one full + one partial, the partial slice
+# in each position of the three-stage ring, tiles that stick out in M, in N and in both.
+@pytest.mark.parametrize("shape", [(300, 200, 72), (257, 132, 32), (100, 260, 40), (129, 64, 100),
+                                   (513, 388, 116), (64, 64, 36), (1, 4, 32), (700, 4, 132),
+                                   (250, 1000, 176), (384, 256, 80)])
+@pytest.mark.parametrize("sched", [None, SCHEDS[2], SCHEDS[3], SCHEDS[4], SCHEDS[5], SCHEDS[6]])
+def test_ragged_shapes_direct_load(oracle, dev, shape, sched):
+    import ctypes
+    from kernelcodegen_amd import lib, ops
+    M, N, K = shape
+    info = lib.LaunchInfo()
+    sp = ctypes.byref(lib.GemmSched(**sched)) if sched else None
+    lib.check(lib.load().kcg_gemm_f32_query(M, N, K, sp, ctypes.byref(info)))
+    bk = int(info.kernel.decode().split("_")[2].split("x")[2])
+    full = b"_dl" in info.kernel and b"ragged" not in info.kernel
+    assert full or (b"_dl_ragged" in info.kernel) == (K >= bk)
+    A = inputs.normal((M, K), 104, 0)
+    B = inputs.normal((K, N), 104, 1)
+    ref = oracle.matmul(A, B)
+    for relu in (False, True):
+        C = ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=relu, sched=sched).cpu().numpy()
+        assert max(rel_err(C, oracle.relu(ref) if relu else ref)) < TOL, (info.kernel, relu)
+
+
+def test_ragged_output_is_not_touched_outside_c(dev):
+    """The clamped edge tiles compute rows and columns that do not exist; none of it may be
+    stored: C sits inside a larger buffer whose other bytes must keep their values."""
+    import torch
+    from kernelcodegen_amd import ops
+    M, N, K = 300, 200, 72
+    A = torch.randn(M, K, device=dev)
+    B = torch.randn(K, N, device=dev)
+    guard = 4096
+    buf = torch.full((M * N + 2 * guard,), 7.0, device=dev)
+    C = buf[guard:guard + M * N].view(M, N)
+    ops.matmul(A, B, relu=True, out=C)
+    assert bool((buf[:guard] == 7.0).all()) and bool((buf[guard + M * N:] == 7.0).all())
+    assert torch.allclose(C, torch.relu(A @ B), rtol=1e-4, atol=1e-3)
+
+
 def test_exact_closed_forms(dev):
     import torch
     from kernelcodegen_amd import ops
