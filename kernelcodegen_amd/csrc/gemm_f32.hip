@@ -307,26 +307,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 #define KCG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define KCG_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
-// One wave-wide direct load: lane l's 16 bytes at (uniform base + off) go to LDS byte
-// address lds_addr + 16 * l.  Issued from assembly so that the address is formed by the
-// instruction itself (scalar base + 32-bit lane offset); the intrinsic materialises a
-// 64-bit address per lane with VALU work, which on this chip comes out of fp32 MFMA time.
-// M0 (the LDS base of the load) is saved and restored around the instruction.
-__device__ __forceinline__ void direct_load_16B(const void *base, unsigned off, unsigned lds_addr) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  unsigned saved_m0;
-  asm volatile(
-      "s_mov_b32 %0, m0\n\t"
-      "s_mov_b32 m0, %1\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %2, %3\n\t"
-      "s_mov_b32 m0, %0"
-      : "=&s"(saved_m0)
-      : "s"(lds_addr), "v"(off), "s"(base)
-      : "memory");
-#endif
-}
-
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 struct GemmDlTile {
   static constexpr int kWaves = WAVES_M * WAVES_N;

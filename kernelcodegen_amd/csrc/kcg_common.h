@@ -39,6 +39,26 @@ __device__ __forceinline__ float relu_maxf(float x) {
   return (x > 0.0f || x != x) ? x : 0.0f;
 }
 
+// One wave-wide direct load: lane l's 16 bytes at (uniform base + off) go to LDS byte
+// address lds_addr + 16 * l.  Issued from assembly so that the address is formed by the
+// instruction itself (scalar base + 32-bit lane offset); the intrinsic materialises a
+// 64-bit address per lane with VALU work, which on this chip comes out of fp32 MFMA time.
+// M0 (the LDS base of the load) is saved and restored around the instruction.
+__device__ __forceinline__ void direct_load_16B(const void *base, unsigned off, unsigned lds_addr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  unsigned saved_m0;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %2, %3\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0)
+      : "s"(lds_addr), "v"(off), "s"(base)
+      : "memory");
+#endif
+}
+
 // Launches `kern` and reports the launch's own status.  hipLaunchKernel returns
 // the error of this launch; hipGetLastError would also surface a stale error
 // left behind by an unrelated earlier runtime call of the host program.
