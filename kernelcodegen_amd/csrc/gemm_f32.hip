@@ -329,7 +329,7 @@ struct GemmDlTile {
   static constexpr int kInstrB = kRunsB / kWaves;
   static constexpr int kSteps = BK / 2;
   static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tile");
-  static_assert(BK == 16 || BK == 32, "K slice");
+  static_assert(BK == 8 || BK == 16 || BK == 32, "K slice");
   static_assert(BN == 64 || BN == 128 || BN == 256, "B rows per run");
   static_assert(kFloatsA % (256 * kWaves) == 0 && kRunsB % kWaves == 0, "load split");
   __host__ __device__ static constexpr int fa(int row) {
@@ -647,7 +647,7 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
     info->lds_bytes = T::kLdsBytes;
     info->waves_per_block = WAVES_M * WAVES_N;
     const char *kind = "";
-    if constexpr (BK == 16 || BK == 32) {
+    if constexpr (BK == 8 || BK == 16 || BK == 32) {
       if ((full || ragged_dl) && K < (1 << 22) && N < (1 << 24)) {
         info->lds_bytes = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>::kLdsBytes;
         kind = full ? "_dl" : "_dl_ragged";
@@ -659,7 +659,7 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
   }
   dim3 grid(static_cast<unsigned>(tiles_m * tiles_n));
   dim3 block(T::kThreads);
-  if constexpr (BK == 16 || BK == 32) {
+  if constexpr (BK == 8 || BK == 16 || BK == 32) {
     using TD = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>;
     // the direct-load kernel addresses a slice with 32-bit byte offsets
     if ((full || ragged_dl) && K < (1 << 22) && N < (1 << 24)) {

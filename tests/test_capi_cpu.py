@@ -74,7 +74,8 @@ def test_launch_geometry_queries():
     s = lib.GemmSched(block_m=128, block_n=128, block_k=8, wave_m=64, wave_n=64)
     assert L.kcg_gemm_f32_query(4096, 2048, 1024, ctypes.byref(s), ctypes.byref(info)) == 0
     assert info.grid[0] == 32 * 16 and info.block[0] == 256
-    assert info.lds_bytes == 2 * (128 * 12 + 8 * 136) * 4
+    # three LDS stages of the direct-load kernel: A 128 x 8, B as four 1 KiB runs 64 B apart
+    assert info.lds_bytes == 3 * (128 * 8 + 4 * 272) * 4 and info.kernel.endswith(b"_dl")
     assert L.kcg_gemm_f32_query(4096, 4096, 4096, None, ctypes.byref(info)) == 0
     assert info.grid[0] * 256 * 128 == 4096 * 4096 and info.lds_bytes <= 160 * 1024
     assert L.kcg_gemm_f32_query(100, 100, 100, None, None) == 1
