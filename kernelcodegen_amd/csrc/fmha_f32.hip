@@ -17,8 +17,7 @@
 //    per tile for the max, one at the end for the sum).
 //  * Q (pre-multiplied by scale * log2 e) stays in registers for the whole sweep
 //    (the reference re-reads it per K/V tile, src/Optimizer/Optimizer.cc:1206).
-//  * K and V tiles are staged in padded LDS in their global layout; the next
-//    tile's global loads are issued before the MFMA phase that hides them
+//  * K and V tiles are fetched directly into LDS before the MFMA phase that hides them
 //    (V_t during S = K_t.Q, K_{t+1} during O += P.V_t).
 //  * The running maximum is a lazily raised reference (see kTau): VALU work between
 //    the two MFMA phases costs matrix time, so the rescale of O is skipped whenever
@@ -26,9 +25,17 @@
 //  * Causal: a workgroup runs the query-block pair (n-1-i, i), so all workgroups
 //    sweep the same number of tiles.
 //
-// LDS (floats): Ks[Bc][D+4]  (b128 reads of 16 consecutive rows hit 64 banks)
-//               Vs[Bc][D+8]  (rows 4 apart are 32 banks apart: the two halves of
-//                             a wave read rows k and k+4 of one column block)
+// K and V tiles go from global memory straight into LDS (global_load_lds_dwordx4 with a
+// scalar base and a 32-bit lane offset: no staging registers, no LDS stores and no address
+// arithmetic on the vector ALU, whose time comes out of the fp32 MFMA's).  An instruction
+// fills 1 KiB of consecutive LDS, lane L supplying the 16 bytes at position L, so rows
+// cannot be padded; each lane fetches whichever global chunk belongs at its position:
+//   Ks: D/32 panels, panel g = [Bc rows][32 floats d = 32g..32g+31]; the 16-byte chunk c
+//       of row r sits at position c ^ ((r >> 1) & 7): the ds_read_b128 of 16 consecutive
+//       rows of one chunk column then hits 16 distinct 16-byte slots of a 256-byte window.
+//   Vs: [Bc rows][D floats]; the 32-float group i of row r sits at group i ^ ((r >> 2) & 1):
+//       rows k and k+4, read together by the two halves of a wave, use different halves
+//       of the 256-byte window.
 #include "kcg_common.h"
 
 namespace kcg {
@@ -37,14 +44,17 @@ template <int D, int BC, int WAVES>
 struct FmhaF32Tile {
   static constexpr int kThreads = 64 * WAVES;
   static constexpr int kBr = 32 * WAVES;
-  static constexpr int kPitchK = D + 4;
-  static constexpr int kPitchV = D + 8;
-  static constexpr int kLdsBytes = (BC * kPitchK + BC * kPitchV) * 4;
-  static constexpr int kLoads = BC * D / 4 / kThreads;  // float4 per thread per tile
+  static constexpr int kTileBytes = BC * D * 4;              // one K (or V) tile, unpadded
+  static constexpr int kLdsBytes = 2 * kTileBytes;
+  static constexpr int kRuns = kTileBytes / 1024;            // 1 KiB direct loads per tile
+  static constexpr int kRunsPerWave = kRuns / WAVES;
+  static constexpr int kPanelBytes = BC * 128;               // K: BC rows x 32 floats of one d-group
+  static constexpr int kRunsPerPanel = BC / 8;
+  static constexpr int kRowsPerRunV = 256 / D;               // V: whole rows per 1 KiB
   static constexpr int kKeyTiles = BC / 32;
   static constexpr int kDTiles = D / 32;
-  static_assert(BC % 32 == 0 && D % 32 == 0, "tile extents");
-  static_assert((BC * D / 4) % kThreads == 0, "load split");
+  static_assert(BC % 32 == 0 && D % 32 == 0 && D <= 256, "tile extents");
+  static_assert(kRuns % WAVES == 0, "load split");
 };
 
 // How far (in log2 units) a tile's row maximum may exceed the running reference before
@@ -79,8 +89,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
                                                           int q_blocks, int q_items, float scale_log2e) {
   using T = FmhaF32Tile<D, BC, WAVES>;
   extern __shared__ __align__(16) float lds[];
-  float *Ks = lds;
-  float *Vs = lds + BC * T::kPitchK;
+  const char *Ks = reinterpret_cast<const char *>(lds);
+  const char *Vs = Ks + T::kTileBytes;
+  const unsigned lds_k = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));  // LDS byte address
+  const unsigned lds_v = lds_k + T::kTileBytes;
 
   // Every XCD walks a contiguous range of (head, work item) ids, head-major, so the
   // K/V of a head are fetched into one XCD's L2 only.  Causal: a work item is the pair
@@ -93,7 +105,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31;
   const int half = lane >> 5;
 
@@ -104,36 +116,63 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
   float *Ob = O + base;
 
 
-  // Tile transfer: thread -> (row ld_row + i * kRowsPerIter, 16-byte column ld_c4).  A full
-  // tile is fetched with a uniform base (scalar registers) plus one per-lane byte offset;
-  // only the ragged last tile pays for per-row predicates (rows at and beyond S read as 0).
-  constexpr int kRowsPerIter = T::kThreads / (D / 4);
-  const int ld_row = tid / (D / 4);
-  const int ld_c4 = tid % (D / 4);
-  const unsigned ld_off = static_cast<unsigned>(ld_row * D + ld_c4 * 4) * 4u;
-  float4_t stage[T::kLoads];
-  auto load_tile = [&](const float *src, int kv0) {
-    const char *g = reinterpret_cast<const char *>(src + static_cast<int64_t>(kv0) * D);
-    if (kv0 + BC <= S) {
+  // ---- direct tile loads ----
+  // Run rho = wave * kRunsPerWave + i of a tile.  K: panel g = rho / kRunsPerPanel, rows
+  // 8q .. 8q+7 (q = rho % kRunsPerPanel); lane L is row 8q + L/8, position L%8.  V: rows
+  // rho * kRowsPerRunV ..; lane L is row + L / (D/4), position L % (D/4).
+  int k_row[T::kRunsPerWave], v_row[T::kRunsPerWave];      // tile row this lane fetches
+  unsigned k_col[T::kRunsPerWave], v_col[T::kRunsPerWave];  // byte offset inside the global row
 #pragma unroll
-      for (int i = 0; i < T::kLoads; ++i)
-        stage[i] = *reinterpret_cast<const float4_t *>(g + i * (kRowsPerIter * D * 4) + ld_off);
-    } else {
+  for (int i = 0; i < T::kRunsPerWave; ++i) {
+    const int rho = wave * T::kRunsPerWave + i;
+    const int g = rho / T::kRunsPerPanel, q = rho % T::kRunsPerPanel;
+    k_row[i] = 8 * q + lane / 8;
+    k_col[i] = static_cast<unsigned>(g * 8 + ((lane % 8) ^ ((k_row[i] >> 1) & 7))) * 16u;
+    v_row[i] = rho * T::kRowsPerRunV + lane / (D / 4);
+    const int pc = lane % (D / 4);
+    v_col[i] = static_cast<unsigned>((((pc >> 3) ^ ((v_row[i] >> 2) & 1)) << 3) + (pc & 7)) * 16u;
+  }
+  // A tile that sticks out beyond S fetches row S-1 in place of the rows that do not exist
+  // (K: those scores are masked; V: those rows are zeroed below before anybody reads them).
+  auto load_k = [&](int kv0) {
+    const char *g = reinterpret_cast<const char *>(Kb + static_cast<int64_t>(kv0) * D);
+    const int last = S - 1 - kv0;
 #pragma unroll
-      for (int i = 0; i < T::kLoads; ++i) {
-        float4_t v = {0.f, 0.f, 0.f, 0.f};
-        if (kv0 + ld_row + i * kRowsPerIter < S)
-          v = *reinterpret_cast<const float4_t *>(g + i * (kRowsPerIter * D * 4) + ld_off);
-        stage[i] = v;
-      }
+    for (int i = 0; i < T::kRunsPerWave; ++i) {
+      const int row = k_row[i] < last ? k_row[i] : last;
+      direct_load_16B(g, static_cast<unsigned>(row) * (D * 4u) + k_col[i],
+                      lds_k + (wave * T::kRunsPerWave + i) * 1024u);
     }
   };
-  auto store_tile = [&](float *dst, int pitch) {
-    float *d = dst + ld_row * pitch + ld_c4 * 4;
+  auto load_v = [&](int kv0) {
+    const char *g = reinterpret_cast<const char *>(Vb + static_cast<int64_t>(kv0) * D);
+    const int last = S - 1 - kv0;
 #pragma unroll
-    for (int i = 0; i < T::kLoads; ++i)
-      *reinterpret_cast<float4_t *>(d + i * kRowsPerIter * pitch) = stage[i];
+    for (int i = 0; i < T::kRunsPerWave; ++i) {
+      const int row = v_row[i] < last ? v_row[i] : last;
+      direct_load_16B(g, static_cast<unsigned>(row) * (D * 4u) + v_col[i],
+                      lds_v + (wave * T::kRunsPerWave + i) * 1024u);
+    }
   };
+  // Waits for this wave's direct loads; V rows at and beyond S become zeros (P is 0 there,
+  // but 0 * inf would not be).
+  auto v_landed = [&](int kv0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (kv0 + BC > S) {
+#pragma unroll
+      for (int i = 0; i < T::kRunsPerWave; ++i)
+        if (kv0 + v_row[i] >= S)
+          *reinterpret_cast<float4_t *>(lds + T::kTileBytes / 4 + (wave * T::kRunsPerWave + i) * 256 + lane * 4) =
+              float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  // per-lane read addresses (bytes inside a tile), swizzles folded in
+  int ka[4];  // K chunk 2j + half of row r32, j = kk % 4 (panel kk / 4 and key tile by offset)
+#pragma unroll
+  for (int j = 0; j < 4; ++j) ka[j] = r32 * 128 + 16 * ((2 * j + half) ^ ((r32 >> 1) & 7));
+  // V[key][32 i + r32] with key = 4 half + (compile-time part): group i ^ half
+  const int va_even = half * (4 * D * 4) + half * 128 + r32 * 4;   // even i: (i ^ half) = i + half
+  const int va_odd = half * (4 * D * 4) - half * 128 + r32 * 4;    // odd i:  (i ^ half) = i - half
 
 #pragma unroll 1
   for (int pass = 0; pass < npass; ++pass) {
@@ -165,13 +204,13 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
   const int kv_end = CAUSAL ? ((q0 + T::kBr) < S ? (q0 + T::kBr) : S) : S;
   const int n_tiles = (kv_end + BC - 1) / BC;
 
-  load_tile(Kb, 0);
-  store_tile(Ks, T::kPitchK);
+  load_k(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   for (int t = 0; t < n_tiles; ++t) {
     const int kv0 = t * BC;
-    load_tile(Vb, kv0);
+    load_v(kv0);
 
     // ---- S^T = K . Q^T  (rows = keys, columns = queries) ----
     float16_t s[T::kKeyTiles];
@@ -179,14 +218,16 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
     for (int kt = 0; kt < T::kKeyTiles; ++kt) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[kt][e] = 0.0f;
-      const float *kp = Ks + (kt * 32 + r32) * T::kPitchK + 4 * half;
       // the K fragment of the next 8 d-columns is requested before the four MFMAs of the
       // current one are issued
+      auto k_frag = [&](int kk) {
+        return *reinterpret_cast<const float4_t *>(Ks + ka[kk % 4] + (kk / 4) * T::kPanelBytes + kt * 32 * 128);
+      };
       float4_t kf[2];
-      kf[0] = *reinterpret_cast<const float4_t *>(kp);
+      kf[0] = k_frag(0);
 #pragma unroll
       for (int kk = 0; kk < D / 8; ++kk) {
-        if (kk + 1 < D / 8) kf[(kk + 1) & 1] = *reinterpret_cast<const float4_t *>(kp + 8 * (kk + 1));
+        if (kk + 1 < D / 8) kf[(kk + 1) & 1] = k_frag(kk + 1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -240,11 +281,11 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
       }
     l_run += psum;
 
-    store_tile(Vs, T::kPitchV);
+    v_landed(kv0);
     __syncthreads();  // V tile visible; every wave is done reading Ks
 
     const bool more = (t + 1) < n_tiles;
-    if (more) load_tile(Kb, kv0 + BC);
+    if (more) load_k(kv0 + BC);
 
     // ---- O^T += V^T . P^T  (rows = d, columns = queries, contraction over keys) ----
     // The matrix phase with the longer dependency chains gets the higher wave priority:
@@ -257,9 +298,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
       float vf[2][T::kDTiles];
       auto vfetch = [&](int x) {
         const int kt = x / 16, e = x % 16;
-        const float *vp = Vs + (kt * 32 + 8 * (e / 4) + 4 * half + (e % 4)) * T::kPitchV + r32;
+        const int row_off = (kt * 32 + 8 * (e / 4) + (e % 4)) * (D * 4);  // + 4 * half rows, in va_*
 #pragma unroll
-        for (int i = 0; i < T::kDTiles; ++i) vf[x & 1][i] = vp[i * 32];
+        for (int i = 0; i < T::kDTiles; ++i)
+          vf[x & 1][i] = *reinterpret_cast<const float *>(Vs + ((i & 1) ? va_odd : va_even) + row_off + i * 128);
       };
       vfetch(0);
 #pragma unroll
@@ -274,7 +316,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
     }
 
     __builtin_amdgcn_s_setprio(0);
-    if (more) store_tile(Ks, T::kPitchK);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // next K tile visible; every wave is done reading Vs
   }
 
@@ -332,7 +374,18 @@ static int launch_fmha_f32(const float *Q, const float *K, const float *V, float
 int dispatch_fmha_f32(const float *Q, const float *K, const float *V, float *O, int B, int H, int S,
                       int D, float scale, int causal, const kcg_fmha_sched *sched,
                       hipStream_t stream, kcg_launch_info *info) {
+  // Default block: 128 query rows (two workgroups per CU).  When that would put exactly one
+  // or two workgroups on every CU for the whole launch, the older workgroup of a CU outruns
+  // the younger and the launch waits for the stragglers: one 256-row workgroup per CU is
+  // faster there (configs[3]: 139 against 136 TFLOP/s) as long as it still fills the chip.
   int br = 128, bc = 32;
+  {
+    const auto items = [&](int rows) {
+      const int64_t blocks = (static_cast<int64_t>(S) + rows - 1) / rows;
+      return (causal ? (blocks + 1) / 2 : blocks) * B * H;
+    };
+    if (items(128) <= 2 * kNumCu && items(256) >= kNumCu) br = 256;
+  }
   if (sched) {
     if (sched->br) br = sched->br;
     if (sched->bc) bc = sched->bc;

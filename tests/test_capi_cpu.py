@@ -88,8 +88,14 @@ def test_launch_geometry_queries():
     assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 0, ctypes.byref(s128), ctypes.byref(info)) == 0
     assert info.grid[0] == 4 * 32 * 32 and info.lds_bytes == 2 * 2 * 64 * 128 * 2
     assert L.kcg_fmha_query(0, 1, 32, 2048, 128, 0, None, ctypes.byref(info)) == 0
-    assert info.grid[0] == 32 * 2048 // 128
-    # fp32 causal: 128-row query blocks in pairs; the 8-wave workgroup is a schedule option
+    # fp32, one workgroup per CU fills the chip exactly: the default is the 256-row workgroup ...
+    assert info.grid[0] == 32 * 2048 // 256 and info.block[0] == 512
+    # ... and the 128-row one where that leaves more (or fewer) workgroups than that
+    assert L.kcg_fmha_query(0, 2, 32, 2048, 128, 0, None, ctypes.byref(info)) == 0
+    assert info.grid[0] == 2 * 32 * 2048 // 128 and info.block[0] == 256
+    assert L.kcg_fmha_query(0, 1, 8, 2048, 128, 0, None, ctypes.byref(info)) == 0
+    assert info.grid[0] == 8 * 2048 // 128 and info.block[0] == 256
+    # fp32 causal: 128-row query blocks in pairs
     assert L.kcg_fmha_query(0, 1, 32, 2048, 128, 1, None, ctypes.byref(info)) == 0
     assert info.grid[0] == 32 * 8 and b"causal_paired" in info.kernel
     s256 = lib.FmhaSched(br=256, bc=32)
