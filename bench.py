@@ -24,7 +24,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 # HBM bytes per launch (fetch + write) measured with rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE, each scaled by the same counter's reading for a 256 MiB copy
 # (profiles/gemm_f32_cfg1.md, profiles/fmha_f32_cfg3.md, profiles/fmha_bf16_cfg4.md).
-TRAFFIC_BYTES = {"gemm_cfg1": 744663460, "fmha_cfg3": 134328811, "fmha_cfg4": 795121940}
+TRAFFIC_BYTES = {"gemm_cfg1": 744663460, "fmha_cfg3": 138053321, "fmha_cfg4": 795121940}
 
 
 def _cpu_model():
