@@ -307,7 +307,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 #define KCG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define KCG_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+// TRANS_B: B is given as [N][K] (the 'T' operand of BatchedMatmul, Q.K^T): its tile then
+// has the shape and the LDS layout of the A tile, rows = n.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool TRANS_B = false>
 struct GemmDlTile {
   static constexpr int kWaves = WAVES_M * WAVES_N;
   static constexpr int kThreads = kWaves * kWaveSize;
@@ -321,7 +323,7 @@ struct GemmDlTile {
   static constexpr int kRowsPerRunB = 256 / BN;      // B rows per 1 KiB run (BN <= 256)
   static constexpr int kRunB = 256 + 2048 / BN;      // floats between runs
   static constexpr int kRunsB = BK * BN / 256;
-  static constexpr int kFloatsB = kRunsB * kRunB;
+  static constexpr int kFloatsB = TRANS_B ? BN * BK : kRunsB * kRunB;
   static constexpr int kStageFloats = kFloatsA + kFloatsB;
   static constexpr int kStages = 3;
   static constexpr int kLdsBytes = kStages * kStageFloats * 4;
@@ -348,12 +350,18 @@ struct GemmDlTile {
 // partial K slice is the one place that needs zeros: its direct loads re-fetch the last
 // full slice (never out of range) and the stage is then rewritten through registers, once
 // per tile.
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool RAGGED, int MIN_WAVES>
+// blockIdx.y is the batch index of BatchedMatmul (src/Frontend/Operators.cc:253-420); the
+// three strides are 0 for the plain matmul.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool RAGGED, int MIN_WAVES,
+          bool TRANS_B = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_dl_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
-    int K, int tiles_m, int tiles_n, int group_m) {
-  using T = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>;
+    int K, int tiles_m, int tiles_n, int group_m, int64_t batch_a, int64_t batch_b, int64_t batch_c) {
+  using T = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N, TRANS_B>;
   extern __shared__ __align__(16) float lds[];
+  A += blockIdx.y * batch_a;
+  B += blockIdx.y * batch_b;
+  C += blockIdx.y * batch_c;
 
   const int logical = xcd_contiguous_id(blockIdx.x, tiles_m * tiles_n);
   const int width = group_m * tiles_n;
@@ -397,13 +405,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 #pragma unroll
   for (int i = 0; i < T::kInstrB; ++i) {
     const int idx = (wave * T::kInstrB + i) * 256 + lane * 4;  // float index in the unpadded B tile
-    const int col = idx % BN;
-    const int gcol = RAGGED ? (col < N - n0 ? col : N - n0 - 4) : col;
-    ob[i] = static_cast<unsigned>((idx / BN) * N + gcol) * 4u;
+    if (TRANS_B) {
+      const int row = idx / BK;
+      const int c_log = ((idx % BK) / 4) ^ T::fa(row);
+      const int grow = RAGGED ? (row < N - n0 ? row : N - n0 - 1) : row;
+      ob[i] = static_cast<unsigned>(grow * K + 4 * c_log) * 4u;
+    } else {
+      const int col = idx % BN;
+      const int gcol = RAGGED ? (col < N - n0 ? col : N - n0 - 4) : col;
+      ob[i] = static_cast<unsigned>((idx / BN) * N + gcol) * 4u;
+    }
   }
   const char *ga = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
-  const char *gb = reinterpret_cast<const char *>(B + n0);
-  const int64_t b_step = static_cast<int64_t>(BK) * N * 4;
+  const char *gb = reinterpret_cast<const char *>(TRANS_B ? B + static_cast<int64_t>(n0) * K : B + n0);
+  const int64_t b_step = TRANS_B ? BK * 4 : static_cast<int64_t>(BK) * N * 4;
   constexpr int kLoadsPerSlice = T::kInstrA + T::kInstrB;
   // load l of the slice at (ga, gb) into the stage at float offset stage_off
   auto issue_one = [&](int stage_off, int l) {
@@ -412,7 +427,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       direct_load_16B(ga, oa[l], static_cast<unsigned>(sa));
     } else {
       const int i = l - T::kInstrA;
-      const int sb = lds_base + (stage_off + T::kFloatsA + (wave * T::kInstrB + i) * T::kRunB) * 4;
+      const int sb = lds_base + (stage_off + T::kFloatsA + (wave * T::kInstrB + i) * (TRANS_B ? 256 : T::kRunB)) * 4;
       direct_load_16B(gb, ob[i], static_cast<unsigned>(sb));
     }
   };
@@ -435,20 +450,29 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   // unrolled over the three stages so that no address arithmetic is left in it -- on this
   // chip every VALU instruction between fp32 MFMAs is paid for in matrix time.
   int a_addr[T::kStages][BK / 8];
-  int b_addr[T::kStages];
+  int b_addr[T::kStages][TRANS_B ? BK / 8 : 1];
 #pragma unroll
   for (int st = 0; st < T::kStages; ++st) {
 #pragma unroll
     for (int kk = 0; kk < BK / 8; ++kk)
       a_addr[st][kk] = lds_base + (st * T::kStageFloats + (wm * T::kWaveM + r32) * BK +
                                    4 * ((2 * kk) ^ half ^ T::fa(r32))) * 4;
-    b_addr[st] = lds_base + (st * T::kStageFloats + T::kFloatsA + half * T::brow(4) + wn * T::kWaveN + r32) * 4;
+    if (TRANS_B) {
+#pragma unroll
+      for (int kk = 0; kk < BK / 8; ++kk)
+        b_addr[st][TRANS_B ? kk : 0] = lds_base + (st * T::kStageFloats + T::kFloatsA + (wn * T::kWaveN + r32) * BK +
+                                                   4 * ((2 * kk) ^ half ^ T::fa(r32))) * 4;
+    } else {
+      b_addr[st][0] = lds_base + (st * T::kStageFloats + T::kFloatsA + half * T::brow(4) + wn * T::kWaveN + r32) * 4;
+    }
   }
 
+  // B operand registers: one float per step, or (TRANS_B) one float4 per group of four steps
+  using BFrag = std::conditional_t<TRANS_B, float4_t, float>;
   float4_t fa[2][T::kTilesM];
-  float fb[2][T::kTilesN];
+  BFrag fb[2][T::kTilesN];
   float4_t na[T::kTilesM];
-  float nb[T::kTilesN];
+  BFrag nb[T::kTilesN];
   auto read_a = [&](int stage, int kk, float4_t(&dst)[T::kTilesM]) {
     const int addr = a_addr[stage][kk];
 #pragma unroll
@@ -458,18 +482,34 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
                    : "v"(addr), "n"(i * 32 * BK * 4)
                    : "memory");
   };
-  auto read_b = [&](int stage, int s, float(&dst)[T::kTilesN]) {
-    const int addr = b_addr[stage];
+  // operands of step s; with TRANS_B only every fourth step reads (the whole group of four)
+  auto read_b = [&](int stage, int s, BFrag(&dst)[T::kTilesN]) {
+    if constexpr (TRANS_B) {
+      const int addr = b_addr[stage][s / 4];
 #pragma unroll
-    for (int n = 0; n < T::kTilesN; ++n)
-      asm volatile("ds_read_b32 %0, %1 offset:%2"
-                   : "=v"(dst[n])
-                   : "v"(addr), "n"((T::brow((s / 4) * 8 + s % 4) + n * 32) * 4)
-                   : "memory");
+      for (int n = 0; n < T::kTilesN; ++n)
+        asm volatile("ds_read_b128 %0, %1 offset:%2"
+                     : "=v"(dst[n])
+                     : "v"(addr), "n"(n * 32 * BK * 4)
+                     : "memory");
+    } else {
+      const int addr = b_addr[stage][0];
+#pragma unroll
+      for (int n = 0; n < T::kTilesN; ++n)
+        asm volatile("ds_read_b32 %0, %1 offset:%2"
+                     : "=v"(dst[n])
+                     : "v"(addr), "n"((T::brow((s / 4) * 8 + s % 4) + n * 32) * 4)
+                     : "memory");
+    }
+  };
+  auto b_operand = [&](const BFrag &f, int s) {
+    if constexpr (TRANS_B) return f[s % 4];
+    else return f;
   };
   constexpr int kReadsA = T::kTilesM;  // LDS instructions per read_a / read_b
   constexpr int kReadsB = T::kTilesN;
-  static_assert((T::brow(BK - 1) + BN) * 4 < 65536 && BM * BK * 4 < 65536, "ds_read offset field");
+  static_assert((T::brow(BK - 1) + BN) * 4 < 65536 && BM * BK * 4 < 65536 && BN * BK * 4 < 65536,
+                "ds_read offset field");
 
   // Publishes the slice requested before the newest one: the wave waits for its
   // own loads of that slice and for its LDS reads, then joins the barrier.  A bare
@@ -505,12 +545,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       } else {
         const int i = l - T::kInstrA;
         const int idx = (wave * T::kInstrB + i) * 256 + lane * 4;
-        const int krow = k0 + idx / BN;
-        const int col = idx % BN;
-        const int gcol = n0 + (col < N - n0 ? col : N - n0 - 4);
-        if (krow < K) v = *reinterpret_cast<const float4_t *>(B + static_cast<int64_t>(krow) * N + gcol);
-        *reinterpret_cast<float4_t *>(lds + stage_off + T::kFloatsA + (wave * T::kInstrB + i) * T::kRunB +
-                                      lane * 4) = v;
+        if (TRANS_B) {
+          const int row = idx / BK;
+          const int k = k0 + 4 * (((idx % BK) / 4) ^ T::fa(row));
+          const int grow = n0 + (row < N - n0 ? row : N - n0 - 1);
+          if (k < K) v = *reinterpret_cast<const float4_t *>(B + static_cast<int64_t>(grow) * K + k);
+          *reinterpret_cast<float4_t *>(lds + stage_off + T::kFloatsA + idx) = v;
+        } else {
+          const int krow = k0 + idx / BN;
+          const int col = idx % BN;
+          const int gcol = n0 + (col < N - n0 ? col : N - n0 - 4);
+          if (krow < K) v = *reinterpret_cast<const float4_t *>(B + static_cast<int64_t>(krow) * N + gcol);
+          *reinterpret_cast<float4_t *>(lds + stage_off + T::kFloatsA + (wave * T::kInstrB + i) * T::kRunB +
+                                        lane * 4) = v;
+        }
       }
     }
   };
@@ -574,10 +622,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       if (s + 1 < T::kSteps) {
         const bool with_a = (s + 1) % 4 == 0;
         if (with_a) read_a(ST, (s + 1) / 4, fa[((s + 1) / 4) & 1]);
-        read_b(ST, s + 1, fb[(s + 1) & 1]);
-        // operands of step s were requested one step ago: all but this step's reads
-        if (with_a) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsA + kReadsB) : "memory");
-        else asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsB) : "memory");
+        if constexpr (TRANS_B) {
+          // both operands come in groups of four steps, requested one step before the group
+          if (with_a) read_b(ST, s + 1, fb[((s + 1) / 4) & 1]);
+          if (s % 4 == 0 && s > 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        } else {
+          read_b(ST, s + 1, fb[(s + 1) & 1]);
+          // operands of step s were requested one step ago: all but this step's reads
+          if (with_a) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsA + kReadsB) : "memory");
+          else asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsB) : "memory");
+        }
       } else {
         publish();  // includes lgkmcnt(0): the operands of the last step are in
         read_a(ST1, 0, na);
@@ -588,8 +642,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
       for (int i = 0; i < T::kTilesM; ++i)
 #pragma unroll
         for (int n = 0; n < T::kTilesN; ++n)
-          acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[(s / 4) & 1][i][s % 4], fb[s & 1][n],
-                                                           acc[i][n], 0, 0, 0);
+          acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+              fa[(s / 4) & 1][i][s % 4], b_operand(fb[TRANS_B ? (s / 4) & 1 : s & 1][n], s), acc[i][n], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
     advance_if(kt + 3 < kfull);
@@ -667,7 +721,7 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
         if (!allow_lds(kern, TD::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
         return launch(kern, grid, block, TD::kLdsBytes, stream, A, B, C, static_cast<int>(M),
                       static_cast<int>(N), static_cast<int>(K), static_cast<int>(tiles_m),
-                      static_cast<int>(tiles_n), group_m);
+                      static_cast<int>(tiles_n), group_m, int64_t{0}, int64_t{0}, int64_t{0});
       };
       if (full)
         return relu ? launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, true, false, MIN_WAVES>)
@@ -694,44 +748,49 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
 #undef KCG_LAUNCH
 }
 
+// Default tile by problem size.  Workgroups are spread over 256 CUs and the CU
+// with the most workgroups sets the run time, so a tile is scored by
+//   (its measured large-problem efficiency) x (tiles / (256 * max tiles per CU));
+// small or awkwardly sized problems thereby get smaller tiles instead of leaving
+// most of the chip idle (the reference's fixed 128x128 tile does the latter).
+static kcg_gemm_sched default_tile(int64_t M, int64_t N, int64_t batch) {
+  kcg_gemm_sched d = {256, 128, 16, 8, 64, 64, 4, 64};
+  struct Cand {
+    int bm, bn, bk, wm, wn;
+    double eff;
+    double max_tiles;  // small tiles re-read A and B too often once the problem outgrows the L2s
+  };
+  // efficiencies measured on problems that fill the chip evenly (fraction of MFMA peak)
+  const Cand cands[] = {{256, 128, 16, 64, 64, 0.91, 1e30},
+                        {128, 128, 32, 64, 64, 0.885, 1e30},  // BLOCK_K 16 is 10 % slower at 4096^3
+                        {128, 64, 32, 64, 32, 0.85, 4096},
+                        {64, 64, 32, 32, 32, 0.84, 6400}};
+  double best = -1.0;
+  for (const Cand &c : cands) {
+    const double per_matrix = static_cast<double>((M + c.bm - 1) / c.bm) * static_cast<double>((N + c.bn - 1) / c.bn);
+    if (per_matrix > c.max_tiles) continue;
+    const double tiles = per_matrix * static_cast<double>(batch);
+    const double per_cu = static_cast<double>((static_cast<int64_t>(tiles) + kNumCu - 1) / kNumCu);
+    // padding waste of ragged edges counts against a large tile too
+    const double useful = (static_cast<double>(M) * N) / (per_matrix * c.bm * c.bn);
+    // a CU left with a single 4-wave workgroup has one wave per SIMD to hide latency with
+    const double lonely = (c.bm * c.bn <= 128 * 128 && tiles <= kNumCu) ? 0.95 : 1.0;
+    const double score = c.eff * lonely * useful * tiles / (per_cu * kNumCu);
+    if (score > best) {
+      best = score;
+      d = {c.bm, c.bn, c.bk, 8, c.wm, c.wn, 4, 64};
+    }
+  }
+  return d;
+}
+
 // Resolves a schedule (NULL / zero fields = defaults) to one of the built tile
 // shapes and either launches it or fills `info`.
 static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
                          int epilogue, const kcg_gemm_sched *s, hipStream_t stream,
                          kcg_launch_info *info) {
-  // Default tile by problem size.  Workgroups are spread over 256 CUs and the CU
-  // with the most workgroups sets the run time, so a tile is scored by
-  //   (its measured large-problem efficiency) x (tiles / (256 * max tiles per CU));
-  // small or awkwardly sized problems thereby get smaller tiles instead of leaving
-  // most of the chip idle (the reference's fixed 128x128 tile does the latter).
   kcg_gemm_sched d = {256, 128, 16, 8, 64, 64, 4, 64};
-  if (!s || (s->block_m == 0 && s->block_n == 0)) {
-    struct Cand {
-      int bm, bn, bk, wm, wn;
-      double eff;
-      double max_tiles;  // small tiles re-read A and B too often once the problem outgrows the L2s
-    };
-    // efficiencies measured on problems that fill the chip evenly (fraction of MFMA peak)
-    const Cand cands[] = {{256, 128, 16, 64, 64, 0.91, 1e30},
-                          {128, 128, 32, 64, 64, 0.885, 1e30},  // BLOCK_K 16 is 10 % slower at 4096^3
-                          {128, 64, 32, 64, 32, 0.85, 4096},
-                          {64, 64, 32, 32, 32, 0.84, 6400}};
-    double best = -1.0;
-    for (const Cand &c : cands) {
-      const double tiles = static_cast<double>((M + c.bm - 1) / c.bm) * static_cast<double>((N + c.bn - 1) / c.bn);
-      if (tiles > c.max_tiles) continue;
-      const double per_cu = static_cast<double>((static_cast<int64_t>(tiles) + kNumCu - 1) / kNumCu);
-      // padding waste of ragged edges counts against a large tile too
-      const double useful = (static_cast<double>(M) * N) / (tiles * c.bm * c.bn);
-      // a CU left with a single 4-wave workgroup has one wave per SIMD to hide latency with
-      const double lonely = (c.bm * c.bn <= 128 * 128 && tiles <= kNumCu) ? 0.95 : 1.0;
-      const double score = c.eff * lonely * useful * tiles / (per_cu * kNumCu);
-      if (score > best) {
-        best = score;
-        d = {c.bm, c.bn, c.bk, 8, c.wm, c.wn, 4, 64};
-      }
-    }
-  }
+  if (!s || (s->block_m == 0 && s->block_n == 0)) d = default_tile(M, N, 1);
   if (s) {
     if (s->block_m) d.block_m = s->block_m;
     if (s->block_n) d.block_n = s->block_n;
@@ -757,6 +816,51 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
   KCG_TRY(128, 64, 32, 2, 2, 2)
 #undef KCG_TRY
   return KCG_ERR_BAD_SCHEDULE;
+}
+
+// BatchedMatmul (src/Frontend/Operators.cc:253-420) on the direct-load kernel: A row-major
+// [batch][M][K]; B [batch][K][N] or, trans_b, [batch][N][K].  Returns
+// KCG_ERR_UNSUPPORTED_SHAPE for problems this kernel does not take (rows that are not
+// 16-byte aligned, K shorter than one slice, more than 65535 matrices).
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MIN_WAVES>
+static int launch_bmm_dl(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N,
+                         int64_t K, bool trans_b, hipStream_t stream) {
+  const int64_t tiles_m = (M + BM - 1) / BM;
+  const int64_t tiles_n = (N + BN - 1) / BN;
+  if (tiles_m * tiles_n > 0x7fffffffLL || M > 0x7fffffffLL || N >= (1 << 24) || K >= (1 << 22) || batch > 65535)
+    return KCG_ERR_UNSUPPORTED_SHAPE;
+  if (K % 4 != 0 || K < BK || (!trans_b && N % 4 != 0) || !aligned16(A) || !aligned16(B))
+    return KCG_ERR_UNSUPPORTED_SHAPE;
+  const bool full = (M % BM == 0) && (N % BN == 0) && (K % BK == 0);
+  dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(batch));
+  dim3 block(WAVES_M * WAVES_N * kWaveSize);
+  auto go = [&](auto kern, int lds_bytes) {
+    if (!allow_lds(kern, lds_bytes)) return static_cast<int>(KCG_ERR_LAUNCH);
+    return launch(kern, grid, block, lds_bytes, stream, A, B, C, static_cast<int>(M), static_cast<int>(N),
+                  static_cast<int>(K), static_cast<int>(tiles_m), static_cast<int>(tiles_n), 8, M * K, K * N,
+                  M * N);
+  };
+  if (trans_b) {
+    constexpr int lds_bytes = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N, true>::kLdsBytes;
+    return full ? go(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, false, MIN_WAVES, true>, lds_bytes)
+                : go(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, true, MIN_WAVES, true>, lds_bytes);
+  }
+  constexpr int lds_bytes = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N, false>::kLdsBytes;
+  return full ? go(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, false, MIN_WAVES, false>, lds_bytes)
+              : go(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, true, MIN_WAVES, false>, lds_bytes);
+}
+
+int dispatch_bmm_dl(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                    bool trans_b, hipStream_t stream) {
+  const kcg_gemm_sched d = default_tile(M, N, batch);
+  if (d.block_m == 256) return launch_bmm_dl<256, 128, 16, 4, 2, 2>(A, B, C, batch, M, N, K, trans_b, stream);
+  // 128 x 128: the shallow slice has the shorter prologue, which is what counts for the short K
+  // of attention products (K = 128: 116 against 107 TFLOP/s); from K = 4096 on the deep one wins
+  if (d.block_m == 128 && d.block_n == 128)
+    return K <= 1024 ? launch_bmm_dl<128, 128, 16, 2, 2, 2>(A, B, C, batch, M, N, K, trans_b, stream)
+                     : launch_bmm_dl<128, 128, 32, 2, 2, 2>(A, B, C, batch, M, N, K, trans_b, stream);
+  if (d.block_m == 128) return launch_bmm_dl<128, 64, 32, 2, 2, 2>(A, B, C, batch, M, N, K, trans_b, stream);
+  return launch_bmm_dl<64, 64, 32, 2, 2, 2>(A, B, C, batch, M, N, K, trans_b, stream);
 }
 
 }  // namespace kcg

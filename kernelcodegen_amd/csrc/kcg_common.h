@@ -87,6 +87,12 @@ inline bool allow_lds(void (*kern)(KArgs...), int lds_bytes) {
                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) == hipSuccess;
 }
 
+// Defined in gemm_f32.hip: BatchedMatmul with A as [batch][M][K] and B as [batch][K][N] or
+// (trans_b) [batch][N][K] on the direct-load matmul kernel; KCG_ERR_UNSUPPORTED_SHAPE when
+// the problem needs the generic kernel instead.
+int dispatch_bmm_dl(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N,
+                    int64_t K, bool trans_b, hipStream_t stream);
+
 // Defined in fmha_f32.hip / fmha_bf16.hip; `info` != nullptr only fills the launch geometry.
 int dispatch_fmha_f32(const float *Q, const float *K, const float *V, float *O, int B, int H, int S,
                       int D, float scale, int causal, const kcg_fmha_sched *sched,

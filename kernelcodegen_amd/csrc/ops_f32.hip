@@ -86,6 +86,8 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Generic rows (any length, any alignment): three sweeps over the row, the second and
+// third served by the caches.
 __global__ __launch_bounds__(256) void softmax_f32_kernel(float *__restrict__ x, int64_t n) {
   __shared__ float red[4];
   float *row = x + static_cast<int64_t>(blockIdx.x) * n;
@@ -111,6 +113,98 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(float *__restrict__ x,
   for (int64_t i = tid; i < n; i += 256) row[i] = exp2f((row[i] - m_use) * kLog2e) * inv;
 }
 
+// Short rows, up to 256 * NV floats (a multiple of 4, 16-byte aligned): one wave per row, the
+// whole row in registers -- every element is read once and written once, all loads of a
+// row are in flight together, and there is neither LDS nor a barrier.  STREAM marks the
+// accesses non-temporal for tensors that are larger than the last-level cache anyway.
+template <int NV, bool STREAM>
+__global__ __launch_bounds__(256) void softmax_f32_wave_rows_kernel(float *__restrict__ x,
+                                                                    int64_t rows, int n4) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  float4_t *p = reinterpret_cast<float4_t *>(x) + row * n4;
+  constexpr float kLog2e = 1.4426950408889634f;
+  float4_t v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + 64 * i;
+    v[i] = float4_t{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if (c < n4) v[i] = STREAM ? __builtin_nontemporal_load(p + c) : p[c];
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) m = fmaxf(fmaxf(m, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
+  m = wave_max(m);
+  const float m_use = (m == -INFINITY) ? 0.0f : m;
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[i][e] = __builtin_amdgcn_exp2f((v[i][e] - m_use) * kLog2e);
+      sum += v[i][e];
+    }
+  sum = wave_sum(sum);
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + 64 * i;
+    const float4_t r = v[i] * inv;
+    if (c < n4) {
+      if (STREAM) __builtin_nontemporal_store(r, p + c);
+      else p[c] = r;
+    }
+  }
+}
+
+// Rows of up to 1024 * NV floats: one workgroup per row, the row in registers, maximum
+// and sum combined through LDS.
+template <int NV, bool STREAM>
+__global__ __launch_bounds__(256) void softmax_f32_block_row_kernel(float *__restrict__ x, int n4) {
+  __shared__ float red[8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float4_t *p = reinterpret_cast<float4_t *>(x) + static_cast<int64_t>(blockIdx.x) * n4;
+  constexpr float kLog2e = 1.4426950408889634f;
+  float4_t v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = tid + 256 * i;
+    v[i] = float4_t{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if (c < n4) v[i] = STREAM ? __builtin_nontemporal_load(p + c) : p[c];
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) m = fmaxf(fmaxf(m, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
+  m = wave_max(m);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float m_use = (m == -INFINITY) ? 0.0f : m;
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[i][e] = __builtin_amdgcn_exp2f((v[i][e] - m_use) * kLog2e);
+      sum += v[i][e];
+    }
+  sum = wave_sum(sum);
+  if (lane == 0) red[4 + wave] = sum;
+  __syncthreads();
+  sum = (red[4] + red[5]) + (red[6] + red[7]);
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = tid + 256 * i;
+    const float4_t r = v[i] * inv;
+    if (c < n4) {
+      if (STREAM) __builtin_nontemporal_store(r, p + c);
+      else p[c] = r;
+    }
+  }
+}
+
 }  // namespace kcg
 
 extern "C" {
@@ -124,8 +218,14 @@ int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int trans
   if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL || tiles_m * tiles_n > 0x7fffffffLL ||
       batch > 65535)
     return KCG_ERR_BAD_SHAPE;
-  dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(batch));
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // the two layouts of the attention graph (Q.K^T is NT, P.V is NN: test/test.cc:71-90) run
+  // on the direct-load matmul kernel when their rows are 16-byte aligned
+  if (!transA) {
+    const int st = kcg::dispatch_bmm_dl(A, B, C, batch, M, N, K, transB != 0, s);
+    if (st != KCG_ERR_UNSUPPORTED_SHAPE) return st;
+  }
+  dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(batch));
   const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
   const int tn = static_cast<int>(tiles_n);
   if (!transA && !transB) return kcg::launch(kcg::bmm_f32_kernel<false, false>, grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
@@ -137,8 +237,32 @@ int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int trans
 int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream) {
   if (!x) return KCG_ERR_NULL_POINTER;
   if (rows <= 0 || n <= 0 || rows > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
-  return kcg::launch(kcg::softmax_f32_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), x, n);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (n % 4 == 0 && n <= 8192 && kcg::aligned16(x)) {
+    const int n4 = static_cast<int>(n / 4);
+    // a tensor that does not fit the 256 MiB last-level cache is streamed past it
+    const bool stream_past = rows * n * 4 > (int64_t{192} << 20);
+    const dim3 wave_grid(static_cast<unsigned>((rows + 3) / 4)), row_grid(static_cast<unsigned>(rows));
+#define KCG_WAVE_ROWS(NV)                                                                          \
+  return stream_past ? kcg::launch(kcg::softmax_f32_wave_rows_kernel<NV, true>, wave_grid,         \
+                                   dim3(256), 0, s, x, rows, n4)                                   \
+                     : kcg::launch(kcg::softmax_f32_wave_rows_kernel<NV, false>, wave_grid,        \
+                                   dim3(256), 0, s, x, rows, n4)
+#define KCG_BLOCK_ROW(NV)                                                                          \
+  return stream_past ? kcg::launch(kcg::softmax_f32_block_row_kernel<NV, true>, row_grid,          \
+                                   dim3(256), 0, s, x, n4)                                         \
+                     : kcg::launch(kcg::softmax_f32_block_row_kernel<NV, false>, row_grid,         \
+                                   dim3(256), 0, s, x, n4)
+    if (n4 <= 64) KCG_WAVE_ROWS(1);
+    if (n4 <= 128) KCG_WAVE_ROWS(2);
+    if (n4 <= 256) KCG_WAVE_ROWS(4);
+    if (n4 <= 512) KCG_BLOCK_ROW(2);
+    if (n4 <= 1024) KCG_BLOCK_ROW(4);
+    KCG_BLOCK_ROW(8);
+#undef KCG_WAVE_ROWS
+#undef KCG_BLOCK_ROW
+  }
+  return kcg::launch(kcg::softmax_f32_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, s, x, n);
 }
 
 }  // extern "C"

@@ -53,9 +53,13 @@ def matmul(A, B, relu=False, out=None, sched=None):
     return out
 
 
-def relu(x, inplace=False):
+def relu(x, inplace=False, out=None):
     _dev_f32(x, "x")
-    y = x if inplace else torch.empty_like(x)
+    if out is not None:
+        _dev_f32(out, "out")
+        if out.numel() != x.numel():
+            raise ValueError("relu: out must have as many elements as x")
+    y = x if inplace else (out if out is not None else torch.empty_like(x))
     lib.check(lib.load().kcg_relu_f32(_ptr(x), _ptr(y), x.numel(), lib.current_stream()))
     return y
 

@@ -47,7 +47,50 @@ def test_batched_matmul(oracle, dev, ta, tb, dims):
     assert max(rel_err(C, ref)) < 1e-4
 
 
-@pytest.mark.parametrize("shape", [(4, 9, 33), (2, 2, 64, 64), (3, 1000), (5, 1), (2, 5000)])
+# Shapes that the direct-load matmul kernel takes (rows 16-byte aligned, K at least one
+# slice): full tiles, ragged edges, K with 1..7 slices and a partial last one, a B^T whose
+# row count is not a multiple of 4, every default tile of the chooser.
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("dims", [
+    ((2, 2), 256, 128, 128),      # attention-like, full tiles
+    ((3,), 128, 256, 32),         # one slice
+    ((2,), 256, 256, 224),        # seven slices of 32
+    ((5,), 130, 132, 100),        # ragged everywhere, partial last slice
+    ((1, 3), 64, 64, 64),         # smallest tile
+    ((2,), 1, 4, 36),             # one row
+    ((2,), 300, 72, 40),          # N = 72 (multiple of 4 only)
+    ((2,), 96, 77, 64),           # N = 77: only the transposed B is 16-byte aligned per row
+    ((40,), 512, 128, 64),        # many matrices: 256 x 128 tiles
+])
+def test_batched_matmul_direct_load(oracle, dev, tb, dims):
+    from kernelcodegen_amd import ops
+    batch, M, N, K = dims
+    A = inputs.normal(batch + (M, K), 312, 0)
+    B = inputs.normal(batch + ((N, K) if tb else (K, N)), 312, 1)
+    ref = oracle.batched_matmul(A, False, B, tb)
+    C = ops.batched_matmul(_gpu(A, dev), _gpu(B, dev), trans_b=tb).cpu().numpy()
+    assert C.shape == ref.shape
+    assert max(rel_err(C, ref)) < 1e-4
+
+
+def test_batched_matmul_output_is_not_touched_outside_c(dev):
+    """Ragged tiles of the batched kernel store nothing beyond each matrix of C."""
+    import torch
+    from kernelcodegen_amd import ops
+    batch, M, N, K = 3, 130, 132, 100
+    A = torch.randn(batch, M, K, device=dev)
+    Bt = torch.randn(batch, N, K, device=dev)
+    buf = torch.full((batch * M * N + 512,), -7.0, device=dev)
+    C = buf[:batch * M * N].view(batch, M, N)
+    ops.batched_matmul(A, Bt, trans_b=True, out=C)
+    assert bool((buf[batch * M * N:] == -7.0).all())
+    ref = torch.matmul(A.double(), Bt.double().transpose(1, 2))
+    assert float((C.double() - ref).abs().max()) < 1e-3
+
+
+@pytest.mark.parametrize("shape", [(4, 9, 33), (2, 2, 64, 64), (3, 1000), (5, 1), (2, 5000), (7, 4), (9, 256),
+                                   (6, 260), (5, 1024), (3, 1028), (5, 2048), (3, 2052), (2, 4096), (3, 8192),
+                                   (2, 8196), (1, 3, 100)])
 def test_softmax(oracle, dev, shape):
     from kernelcodegen_amd import ops
     x = inputs.normal(shape, 303, 0) * np.float32(2)
@@ -58,6 +101,23 @@ def test_softmax(oracle, dev, shape):
     y = y.cpu().numpy()
     assert max(rel_err(y, ref)) < 1e-4
     assert np.allclose(y.sum(-1), 1, atol=1e-5)
+
+
+def test_softmax_rows_with_large_and_infinite_entries(dev):
+    """x = 100 would overflow exp() in the reference's un-shifted form; the shifted form
+    stays finite.  A row of -inf except one entry is a one-hot."""
+    import torch
+    from kernelcodegen_amd import ops
+    for n in (8, 512, 2048, 6000):
+        x = torch.full((4, n), 100.0, device=dev)
+        x[1] = -float("inf")
+        x[1, n // 2] = 3.0
+        x[2, 0] = 130.0
+        y = ops.softmax_(x.clone())
+        assert torch.allclose(y[0], torch.full((n,), 1.0 / n, device=dev), rtol=1e-5)
+        assert float(y[1, n // 2]) == 1.0 and float(y[1].sum()) == 1.0
+        assert abs(float(y[2, 0]) - 1.0) < 1e-6
+        assert bool(torch.isfinite(y).all())
 
 
 def test_unfused_graph_matches_fused_kernel(oracle, dev):
