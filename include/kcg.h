@@ -144,7 +144,8 @@ KCG_API int kcg_relu_f32(const float *x, float *y, int64_t n, void *stream);
 /* C[b] = op(A[b]) . op(B[b]) for `batch` contiguous matrices.
  * transA = 0: A is [batch,M,K]; 1: [batch,K,M].  transB = 0: B is [batch,K,N];
  * 1: [batch,N,K].  src/Frontend/Operators.cc:253-420 (name suffix _NN/_NT/...,
- * :329-339). */
+ * :329-339).  NN and NT with 16-byte aligned rows (K % 4 == 0, and N % 4 == 0 for
+ * NN) run on the tiled matmul kernel; every other case on a generic kernel. */
 KCG_API int kcg_batched_matmul_f32(const float *A, int transA, const float *B,
                                    int transB, float *C, int64_t batch, int64_t M,
                                    int64_t N, int64_t K, void *stream);
