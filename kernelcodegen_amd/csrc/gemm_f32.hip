@@ -304,9 +304,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 // Three LDS stages: slice kt+2 is requested at the top of slice kt and has two
 // slices of MFMA time to arrive; a wave only waits for its own loads of slice
 // kt+1 (vmcnt) right before the barrier that publishes them.
-#define KCG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
-#define KCG_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
-
 // TRANS_B: B is given as [N][K] (the 'T' operand of BatchedMatmul, Q.K^T): its tile then
 // has the shape and the LDS layout of the A tile, rows = n.
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool TRANS_B = false>

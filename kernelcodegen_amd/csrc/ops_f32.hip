@@ -209,16 +209,10 @@ __global__ __launch_bounds__(256) void softmax_f32_block_row_kernel(float *__res
 
 extern "C" {
 
-int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int transB, float *C,
-                           int64_t batch, int64_t M, int64_t N, int64_t K, void *stream) {
-  if (!A || !B || !C) return KCG_ERR_NULL_POINTER;
-  if (batch <= 0 || M <= 0 || N <= 0 || K <= 0) return KCG_ERR_BAD_SHAPE;
-  if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1)) return KCG_ERR_BAD_ARGUMENT;
+// At most 65535 matrices per launch (grid.y).
+static int batched_matmul_chunk(const float *A, int transA, const float *B, int transB, float *C,
+                                int64_t batch, int64_t M, int64_t N, int64_t K, hipStream_t s) {
   const int64_t tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
-  if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL || tiles_m * tiles_n > 0x7fffffffLL ||
-      batch > 65535)
-    return KCG_ERR_BAD_SHAPE;
-  hipStream_t s = static_cast<hipStream_t>(stream);
   // the two layouts of the attention graph (Q.K^T is NT, P.V is NN: test/test.cc:71-90) run
   // on the direct-load matmul kernel when their rows are 16-byte aligned
   if (!transA) {
@@ -232,6 +226,24 @@ int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int trans
   if (!transA && transB) return kcg::launch(kcg::bmm_f32_kernel<false, true>, grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
   if (transA && !transB) return kcg::launch(kcg::bmm_f32_kernel<true, false>, grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
   return kcg::launch(kcg::bmm_f32_kernel<true, true>, grid, dim3(256), 0, s, A, B, C, m, n, k, tn);
+}
+
+int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int transB, float *C,
+                           int64_t batch, int64_t M, int64_t N, int64_t K, void *stream) {
+  if (!A || !B || !C) return KCG_ERR_NULL_POINTER;
+  if (batch <= 0 || M <= 0 || N <= 0 || K <= 0) return KCG_ERR_BAD_SHAPE;
+  if ((transA != 0 && transA != 1) || (transB != 0 && transB != 1)) return KCG_ERR_BAD_ARGUMENT;
+  if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL ||
+      ((M + 63) / 64) * ((N + 63) / 64) > 0x7fffffffLL)
+    return KCG_ERR_BAD_SHAPE;
+  constexpr int64_t kMaxPerLaunch = 65535;
+  for (int64_t b0 = 0; b0 < batch; b0 += kMaxPerLaunch) {
+    const int64_t nb = batch - b0 < kMaxPerLaunch ? batch - b0 : kMaxPerLaunch;
+    const int st = batched_matmul_chunk(A + b0 * M * K, transA, B + b0 * K * N, transB, C + b0 * M * N, nb,
+                                        M, N, K, static_cast<hipStream_t>(stream));
+    if (st != KCG_OK) return st;
+  }
+  return KCG_OK;
 }
 
 int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream) {

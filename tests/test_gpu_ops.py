@@ -73,6 +73,20 @@ def test_batched_matmul_direct_load(oracle, dev, tb, dims):
     assert max(rel_err(C, ref)) < 1e-4
 
 
+@pytest.mark.parametrize("K", [32, 3])
+def test_batched_matmul_more_matrices_than_one_launch_takes(dev, K):
+    """70000 small matrices: more than the 65535 a launch holds in its grid (K = 32 on the
+    tiled kernel, K = 3 on the generic one)."""
+    import torch
+    from kernelcodegen_amd import ops
+    batch, M, N = 70000, 4, 4
+    A = torch.randn(batch, M, K, device=dev)
+    B = torch.randn(batch, K, N, device=dev)
+    C = ops.batched_matmul(A, B)
+    ref = torch.einsum("bmk,bkn->bmn", A.double(), B.double())
+    assert float((C.double() - ref).abs().max()) < 1e-4
+
+
 def test_batched_matmul_output_is_not_touched_outside_c(dev):
     """Ragged tiles of the batched kernel store nothing beyond each matrix of C."""
     import torch
