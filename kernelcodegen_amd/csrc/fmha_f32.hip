@@ -208,7 +208,14 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  for (int t = 0; t < n_tiles; ++t) {
+  // Causal: the tiles that lie wholly above this wave's 32 query rows contribute nothing
+  // (every P is 0).  The wave computes the first n_own tiles and, in a second loop that
+  // does not touch the accumulators, only moves its share of the remaining tiles and keeps
+  // the barriers; the matrix pipe of its SIMD is then free for the other workgroup of the CU.
+  const int last_row_tile = (q0 + wave * 32 + 31) / BC;
+  const int n_own = (CAUSAL && last_row_tile + 1 < n_tiles) ? last_row_tile + 1 : n_tiles;
+
+  for (int t = 0; t < n_own; ++t) {
     const int kv0 = t * BC;
     load_v(kv0);
 
@@ -318,6 +325,17 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
     __builtin_amdgcn_s_setprio(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // next K tile visible; every wave is done reading Vs
+  }
+  if (CAUSAL) {
+    for (int t = n_own; t < n_tiles; ++t) {
+      const int kv0 = t * BC;
+      load_v(kv0);
+      v_landed(kv0);
+      __syncthreads();
+      if ((t + 1) < n_tiles) load_k(kv0 + BC);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
   }
 
   // ---- normalise and store: lane holds O[qrow][32*i + 8*g + 4*half + 0..3] ----
