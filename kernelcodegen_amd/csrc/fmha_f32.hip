@@ -392,16 +392,15 @@ static int launch_fmha_f32(const float *Q, const float *K, const float *V, float
 int dispatch_fmha_f32(const float *Q, const float *K, const float *V, float *O, int B, int H, int S,
                       int D, float scale, int causal, const kcg_fmha_sched *sched,
                       hipStream_t stream, kcg_launch_info *info) {
-  // Default block: 128 query rows (two workgroups per CU).  When that would put exactly one
-  // or two workgroups on every CU for the whole launch, the older workgroup of a CU outruns
-  // the younger and the launch waits for the stragglers: one 256-row workgroup per CU is
-  // faster there (configs[3]: 139 against 136 TFLOP/s) as long as it still fills the chip.
+  // Default block: 128 query rows (two workgroups per CU).  On a short non-causal sweep that
+  // puts exactly one or two such workgroups on every CU for the whole launch, the older
+  // workgroup of a CU outruns the younger and the launch waits for the stragglers: one
+  // 256-row workgroup per CU is faster there (configs[3]: 139 against 134 TFLOP/s).  On
+  // longer sweeps and on causal launches the small block measures 1-3 % faster, and far
+  // faster whenever the large one would leave CUs idle.
   int br = 128, bc = 32;
-  {
-    const auto items = [&](int rows) {
-      const int64_t blocks = (static_cast<int64_t>(S) + rows - 1) / rows;
-      return (causal ? (blocks + 1) / 2 : blocks) * B * H;
-    };
+  if (!causal && S <= 2048) {
+    const auto items = [&](int rows) { return (static_cast<int64_t>(S) + rows - 1) / rows * B * H; };
     if (items(128) <= 2 * kNumCu && items(256) >= kNumCu) br = 256;
   }
   if (sched) {
