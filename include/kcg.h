@@ -80,7 +80,8 @@ typedef struct kcg_gemm_sched {
  * src/Backend/CUDA.cc:793-801; adaptor contract test/test.cc:27-33).
  * Any M, N, K >= 1 is accepted (the reference requires M, N % 128 == 0 and
  * K % 8 == 0, src/Optimizer/Rewriter.cc:124-128); ragged edges take a
- * bounds-checked path.  A, B, C must not alias. */
+ * bounds-checked path.  A, B, C must not alias.  Each of A, B and C is limited to
+ * 2^31 - 1 elements (8 GiB); beyond that KCG_ERR_UNSUPPORTED_SHAPE is returned. */
 KCG_API int kcg_gemm_f32(const float *A, const float *B, float *C, int64_t M,
                          int64_t N, int64_t K, int epilogue,
                          const kcg_gemm_sched *sched, void *stream);
@@ -115,7 +116,9 @@ typedef struct kcg_fmha_sched {
  * (src/Optimizer/Optimizer.cc:1101-1118); semantics are those of the Frontend
  * graph BatchedMatmul(Q,K^T) -> Softmax(axis -1) -> BatchedMatmul(P,V)
  * (test/test.cc:88-90).  scale = 1 and causal = 0 give exactly that graph;
- * scale and causal are extensions.  D must be 64 or 128; any S >= 1. */
+ * scale and causal are extensions.  D must be 64 or 128; any S >= 1; each tensor is
+ * limited to 2^31 - 1 elements (KCG_ERR_UNSUPPORTED_SHAPE beyond; also for the bf16
+ * entry point and for every operand of kcg_batched_matmul_f32). */
 KCG_API int kcg_fmha_f32(const float *Q, const float *K, const float *V, float *O,
                          int32_t B, int32_t H, int32_t S, int32_t D, float scale,
                          int causal, const kcg_fmha_sched *sched, void *stream);

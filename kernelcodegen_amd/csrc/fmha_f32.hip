@@ -437,6 +437,8 @@ int kcg_fmha_f32(const float *Q, const float *K, const float *V, float *O, int32
   if (!(scale == scale)) return KCG_ERR_BAD_ARGUMENT;
   if (!kcg::aligned16(Q) || !kcg::aligned16(K) || !kcg::aligned16(V) || !kcg::aligned16(O))
     return KCG_ERR_BAD_ARGUMENT;
+  // tensors of 2^31 elements and more: not verified on the GPU (see kcg_gemm_f32)
+  if (static_cast<int64_t>(B) * H > 0x7fffffffLL / (static_cast<int64_t>(S) * D)) return KCG_ERR_UNSUPPORTED_SHAPE;
   return kcg::dispatch_fmha_f32(Q, K, V, O, B, H, S, D, scale, causal, sched,
                                 static_cast<hipStream_t>(stream), nullptr);
 }

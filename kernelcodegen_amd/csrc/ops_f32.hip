@@ -236,6 +236,12 @@ int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int trans
   if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL ||
       ((M + 63) / 64) * ((N + 63) / 64) > 0x7fffffffLL)
     return KCG_ERR_BAD_SHAPE;
+  // tensors of 2^31 elements and more: not verified on the GPU (see kcg_gemm_f32)
+  {
+    const int64_t mk = M * K, kn = K * N, mn = M * N;  // each below 2^62
+    const int64_t largest = mk > kn ? (mk > mn ? mk : mn) : (kn > mn ? kn : mn);
+    if (batch > 0x7fffffffLL / largest) return KCG_ERR_UNSUPPORTED_SHAPE;
+  }
   constexpr int64_t kMaxPerLaunch = 65535;
   for (int64_t b0 = 0; b0 < batch; b0 += kMaxPerLaunch) {
     const int64_t nb = batch - b0 < kMaxPerLaunch ? batch - b0 : kMaxPerLaunch;

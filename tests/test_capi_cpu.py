@@ -112,3 +112,17 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(lib, "LIB_PATH", "/nonexistent/libkcg_hip.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         lib.load()
+
+
+def test_tensors_of_two_to_the_31_elements_are_refused():
+    """The size check comes before any launch or device query, so it runs without a GPU and
+    never touches the (fake) pointers."""
+    L = lib.load()
+    fake = ctypes.c_void_p(256)
+    unsupported = 3
+    assert L.kcg_gemm_f32(fake, fake, fake, 66000, 128, 33000, 0, None, None) == unsupported
+    assert L.kcg_gemm_f32(fake, fake, fake, 66000, 33000, 64, 0, None, None) == unsupported
+    assert L.kcg_gemm_f32(fake, fake, fake, 64, 66000, 33000, 0, None, None) == unsupported
+    assert L.kcg_batched_matmul_f32(fake, 0, fake, 1, fake, 64, 8192, 8192, 128, None) == unsupported
+    assert L.kcg_fmha_f32(fake, fake, fake, fake, 64, 64, 4096, 128, 1.0, 0, None, None) == unsupported
+    assert L.kcg_fmha_bf16(fake, fake, fake, fake, 1, 64, 64, 4096, 128, 1.0, 1, None, None) == unsupported

@@ -237,3 +237,25 @@ def test_bf16_default_schedule_and_large_logits(oracle, dev):
         ref = oracle.fmha(Q, K, V, scale=scale, causal=causal, stable=True, rows=(1990, 2118))
         O = ops.fmha(tq, tk, tv, scale=scale, causal=causal, out_dtype=torch.float32)
         assert max(rel_err(O[:, :, 1990:2118].cpu().numpy(), ref)) < TOL_BF16
+
+
+@pytest.mark.skip(reason="never run: the matmul test of the same size class ended in a GPU memory fault "
+                         "whose cause is not found")
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_tensors_beyond_two_to_the_31_elements(dev, dtype):
+    """Q, K, V, O of 2.15e9 elements each (B=64, H=64, S=4096, D=128): the last heads, whose
+    element offsets exceed 2^31, must equal the same heads run on their own."""
+    import torch
+    from kernelcodegen_amd import ops
+    B, H, S, D = 64, 64, 4096, 128
+    assert B * H * S * D > 2 ** 31
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    Q = torch.empty(B, H, S, D, device=dev, dtype=td).normal_()
+    K = torch.empty_like(Q).normal_()
+    V = torch.empty_like(Q).normal_()
+    O = ops.fmha(Q, K, V, scale=D ** -0.5, causal=True)
+    last = ops.fmha(Q[-1:, -2:].contiguous(), K[-1:, -2:].contiguous(), V[-1:, -2:].contiguous(),
+                    scale=D ** -0.5, causal=True)
+    tol = 2e-2 if dtype == "bf16" else 1e-4
+    assert float((O[-1:, -2:].float() - last.float()).abs().max()) < tol
+    assert bool(torch.isfinite(O[-1].float()).all())
