@@ -26,6 +26,7 @@
 // read of A) and the j-th MFMA of the group consumes k = 4h + j from both
 // operands.  The set of products summed into each C element is unchanged; only
 // their order differs from the ascending-k order of the reference nest.
+#include <cstring>
 #include <type_traits>
 
 #include "kcg_common.h"
@@ -746,58 +747,97 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
 }
 
 // Default tile by problem size.  Workgroups are spread over 256 CUs and the CU
-// with the most workgroups sets the run time, so a tile is scored by
-//   (its measured large-problem efficiency) x (tiles / (256 * max tiles per CU));
+// with the most workgroups sets the run time, so a tile is priced at
+//   (tile area) x (max tiles per CU) / (its measured large-problem efficiency);
 // small or awkwardly sized problems thereby get smaller tiles instead of leaving
 // most of the chip idle (the reference's fixed 128x128 tile does the latter).
-static kcg_gemm_sched default_tile(int64_t M, int64_t N, int64_t batch) {
-  kcg_gemm_sched d = {256, 128, 16, 8, 64, 64, 4, 64};
-  struct Cand {
-    int bm, bn, bk, wm, wn;
-    double eff;
-    double max_tiles;  // small tiles re-read A and B too often once the problem outgrows the L2s
-  };
-  // efficiencies measured on problems that fill the chip evenly (fraction of MFMA peak)
-  const Cand cands[] = {{256, 128, 16, 64, 64, 0.91, 1e30},
-                        {128, 128, 32, 64, 64, 0.885, 1e30},  // BLOCK_K 16 is 10 % slower at 4096^3
-                        {128, 64, 32, 64, 32, 0.85, 4096},
-                        {64, 64, 32, 32, 32, 0.84, 6400}};
+struct TileCand {
+  int bm, bn, bk, wm, wn;
+  double eff;        // fraction of MFMA peak on problems that fill the chip evenly
+  double max_tiles;  // small tiles re-read A and B too often once the problem outgrows the L2s
+};
+static constexpr TileCand kTileCands[] = {{256, 128, 16, 64, 64, 0.91, 1e30},
+                                          {128, 128, 32, 64, 64, 0.885, 1e30},  // BLOCK_K 16 is 10 % slower at 4096^3
+                                          {128, 64, 32, 64, 32, 0.85, 4096},
+                                          {64, 64, 32, 32, 32, 0.84, 6400}};
+
+// Cost of `batch` M x N problems on tile c, in tile-area units per CU (proportional to run
+// time for a given K); negative when the tile is not a candidate for this size.
+static double tile_cost(const TileCand &c, int64_t M, int64_t N, int64_t batch) {
+  const double per_matrix = static_cast<double>((M + c.bm - 1) / c.bm) * static_cast<double>((N + c.bn - 1) / c.bn);
+  if (per_matrix > c.max_tiles) return -1.0;
+  const double tiles = per_matrix * static_cast<double>(batch);
+  const double per_cu = static_cast<double>((static_cast<int64_t>(tiles) + kNumCu - 1) / kNumCu);
+  // a CU left with a single 4-wave workgroup has one wave per SIMD to hide latency with
+  const double lonely = (c.bm * c.bn <= 128 * 128 && tiles <= kNumCu) ? 0.95 : 1.0;
+  return per_cu * c.bm * c.bn / (c.eff * lonely);
+}
+
+static kcg_gemm_sched sched_of(const TileCand &c) { return {c.bm, c.bn, c.bk, 8, c.wm, c.wn, 4, 64}; }
+
+static kcg_gemm_sched default_tile(int64_t M, int64_t N, int64_t batch, double *cost_out = nullptr) {
+  kcg_gemm_sched d = sched_of(kTileCands[0]);
   double best = -1.0;
-  for (const Cand &c : cands) {
-    const double per_matrix = static_cast<double>((M + c.bm - 1) / c.bm) * static_cast<double>((N + c.bn - 1) / c.bn);
-    if (per_matrix > c.max_tiles) continue;
-    const double tiles = per_matrix * static_cast<double>(batch);
-    const double per_cu = static_cast<double>((static_cast<int64_t>(tiles) + kNumCu - 1) / kNumCu);
-    // padding waste of ragged edges counts against a large tile too
-    const double useful = (static_cast<double>(M) * N) / (per_matrix * c.bm * c.bn);
-    // a CU left with a single 4-wave workgroup has one wave per SIMD to hide latency with
-    const double lonely = (c.bm * c.bn <= 128 * 128 && tiles <= kNumCu) ? 0.95 : 1.0;
-    const double score = c.eff * lonely * useful * tiles / (per_cu * kNumCu);
-    if (score > best) {
-      best = score;
-      d = {c.bm, c.bn, c.bk, 8, c.wm, c.wn, 4, 64};
+  for (const TileCand &c : kTileCands) {
+    const double cost = tile_cost(c, M, N, batch);
+    if (cost < 0.0) continue;
+    if (best < 0.0 || cost < best) {
+      best = cost;
+      d = sched_of(c);
     }
   }
+  if (cost_out) *cost_out = best;
   return d;
+}
+
+// A large problem whose tile count leaves the last round of workgroups mostly empty is cut
+// in two along M: the first `main_rows` rows run on the 256 x 128 tile in whole rounds, the
+// rest on a small tile in a second launch on the same stream (rows of a row-major matrix are
+// contiguous, so both are ordinary matmuls on sub-matrices).  7168^3: 140 -> 149 TFLOP/s,
+// 9216^3: 144 -> 151, 3072^3: 125 -> 134.  main_rows == M: one launch.
+struct GemmPlan {
+  kcg_gemm_sched main;
+  int64_t main_rows;
+  kcg_gemm_sched tail;
+};
+static GemmPlan default_plan(int64_t M, int64_t N) {
+  GemmPlan plan;
+  double single = 0.0;
+  plan.main = default_tile(M, N, 1, &single);
+  plan.main_rows = M;
+  plan.tail = plan.main;
+  const TileCand &big = kTileCands[0];
+  const int64_t rows_of_tiles = (M + big.bm - 1) / big.bm;
+  // Worth it only when a few tiles spill into one more round (tiles per CU = n + a small
+  // fraction): workgroups of a launch run nearly in step, so those few hold the whole chip
+  // for a round; with a fraction around one half the measured loss is small (6144^3: 152).
+  const int64_t tiles = rows_of_tiles * ((N + big.bn - 1) / big.bn);
+  const int64_t spill = tiles % kNumCu;
+  if (tiles <= kNumCu || spill == 0 || spill * 20 > kNumCu * 7) return plan;
+  // the model prices the two launches as if the second waited for the last workgroup of the
+  // first at full cost; measured, the cut does better than that by about 5 %
+  constexpr double kSplitBias = 0.95;
+  double best = single;
+  for (int64_t k = 1; k <= 8 && k < rows_of_tiles; ++k) {
+    const int64_t m1 = (rows_of_tiles - k) * big.bm;
+    const double c1 = tile_cost(big, m1, N, 1);
+    double c2 = 0.0;
+    const kcg_gemm_sched t = default_tile(M - m1, N, 1, &c2);
+    const double cost = (c1 + c2) * kSplitBias;
+    if (cost < best) {
+      best = cost;
+      plan.main = sched_of(big);
+      plan.main_rows = m1;
+      plan.tail = t;
+    }
+  }
+  return plan;
 }
 
 // Resolves a schedule (NULL / zero fields = defaults) to one of the built tile
 // shapes and either launches it or fills `info`.
-static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
-                         int epilogue, const kcg_gemm_sched *s, hipStream_t stream,
-                         kcg_launch_info *info) {
-  kcg_gemm_sched d = {256, 128, 16, 8, 64, 64, 4, 64};
-  if (!s || (s->block_m == 0 && s->block_n == 0)) d = default_tile(M, N, 1);
-  if (s) {
-    if (s->block_m) d.block_m = s->block_m;
-    if (s->block_n) d.block_n = s->block_n;
-    if (s->block_k) d.block_k = s->block_k;
-    if (s->group_m) d.group_m = s->group_m;
-    if (s->wave_m) d.wave_m = s->wave_m;
-    if (s->wave_n) d.wave_n = s->wave_n;
-    if (s->vec_width) d.vec_width = s->vec_width;
-    if (s->wave_size) d.wave_size = s->wave_size;
-  }
+static int launch_sched(const kcg_gemm_sched &d, const float *A, const float *B, float *C, int64_t M, int64_t N,
+                        int64_t K, int epilogue, hipStream_t stream, kcg_launch_info *info) {
   if (d.wave_size != 64 || d.vec_width != 4 || d.group_m < 1) return KCG_ERR_BAD_SCHEDULE;
 #define KCG_TRY(BM, BN, BK, WM, WN, MINW)                                                         \
   if (d.block_m == BM && d.block_n == BN && d.block_k == BK && d.wave_m == BM / WM &&             \
@@ -813,6 +853,47 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
   KCG_TRY(128, 64, 32, 2, 2, 2)
 #undef KCG_TRY
   return KCG_ERR_BAD_SCHEDULE;
+}
+
+static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
+                         int epilogue, const kcg_gemm_sched *s, hipStream_t stream,
+                         kcg_launch_info *info) {
+  kcg_gemm_sched d = {256, 128, 16, 8, 64, 64, 4, 64};
+  if (!s || (s->block_m == 0 && s->block_n == 0)) {
+    const GemmPlan plan = default_plan(M, N);
+    d = plan.main;
+    if (plan.main_rows < M) {
+      // caller's remaining fields (GROUP_SIZE_M) apply to both launches
+      kcg_gemm_sched t = plan.tail;
+      if (s && s->group_m) d.group_m = t.group_m = s->group_m;
+      if (s && ((s->wave_size && s->wave_size != 64) || (s->vec_width && s->vec_width != 4)))
+        return KCG_ERR_BAD_SCHEDULE;
+      const int64_t m1 = plan.main_rows;
+      if (info) {
+        // geometry of the main launch; the second launch is named after it
+        const int st = launch_sched(d, A, B, C, m1, N, K, epilogue, stream, info);
+        if (st != KCG_OK) return st;
+        const size_t used = strlen(info->kernel);
+        snprintf(info->kernel + used, sizeof info->kernel - used, "+%lldrows_%dx%dx%d", static_cast<long long>(M - m1),
+                 t.block_m, t.block_n, t.block_k);
+        return KCG_OK;
+      }
+      const int st = launch_sched(d, A, B, C, m1, N, K, epilogue, stream, nullptr);
+      if (st != KCG_OK) return st;
+      return launch_sched(t, A + m1 * K, B, C + m1 * N, M - m1, N, K, epilogue, stream, nullptr);
+    }
+  }
+  if (s) {
+    if (s->block_m) d.block_m = s->block_m;
+    if (s->block_n) d.block_n = s->block_n;
+    if (s->block_k) d.block_k = s->block_k;
+    if (s->group_m) d.group_m = s->group_m;
+    if (s->wave_m) d.wave_m = s->wave_m;
+    if (s->wave_n) d.wave_n = s->wave_n;
+    if (s->vec_width) d.vec_width = s->vec_width;
+    if (s->wave_size) d.wave_size = s->wave_size;
+  }
+  return launch_sched(d, A, B, C, M, N, K, epilogue, stream, info);
 }
 
 // BatchedMatmul (src/Frontend/Operators.cc:253-420) on the direct-load kernel: A row-major

@@ -79,6 +79,15 @@ def test_launch_geometry_queries():
     assert L.kcg_gemm_f32_query(4096, 4096, 4096, None, ctypes.byref(info)) == 0
     assert info.grid[0] * 256 * 128 == 4096 * 4096 and info.lds_bytes <= 160 * 1024
     assert L.kcg_gemm_f32_query(100, 100, 100, None, None) == 1
+    # 7168^3: 1568 large tiles would spill 32 into a seventh round; 27 rows of tiles run in
+    # whole rounds and the last 256 rows of C as a second launch on the 64 x 64 tile
+    assert L.kcg_gemm_f32_query(7168, 7168, 7168, None, ctypes.byref(info)) == 0
+    assert info.grid[0] == 27 * 56 and info.block[0] == 512
+    assert info.kernel == b"gemm_f32_256x128x16_w4x2_dl+256rows_64x64x32"
+    # an explicit tile is never cut
+    s = lib.GemmSched(block_m=256, block_n=128, block_k=16, wave_m=64, wave_n=64)
+    assert L.kcg_gemm_f32_query(7168, 7168, 7168, ctypes.byref(s), ctypes.byref(info)) == 0
+    assert info.grid[0] == 28 * 56 and b"+" not in info.kernel
     # bf16 causal, S = 4096: 256-row query blocks run in pairs (n-1-i, i) -> 8 work items per head
     assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 1, None, ctypes.byref(info)) == 0
     assert info.grid[0] == 4 * 32 * 8 and info.block[0] == 512 and info.waves_per_block == 8

@@ -202,6 +202,27 @@ def test_shape_mismatch_raises(dev):
                    sched=dict(block_m=96))
 
 
+@pytest.mark.parametrize("shape", [(3072, 3072, 96), (4100, 4100, 64), (66000 // 8, 128 * 9, 40), (5120, 5120, 32)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_problems_cut_into_a_main_and_a_tail_launch(oracle, dev, shape, relu):
+    """With no schedule given, a problem whose 256 x 128 tiles spill a little into one more
+    round runs as two launches (whole rounds of the large tile, the last rows on a small
+    tile); the query names both."""
+    import ctypes
+    from kernelcodegen_amd import lib, ops
+    M, N, K = shape
+    info = lib.LaunchInfo()
+    lib.check(lib.load().kcg_gemm_f32_query(M, N, K, None, ctypes.byref(info)))
+    assert b"+" in info.kernel and b"rows_" in info.kernel, info.kernel
+    A = inputs.normal((M, K), 41, 0)
+    B = inputs.normal((K, N), 41, 1)
+    ref = oracle.matmul(A, B)
+    if relu:
+        ref = oracle.relu(ref)
+    C = ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=relu).cpu().numpy()
+    assert max(rel_err(C, ref)) < TOL
+
+
 @pytest.mark.skip(reason="the one run of this case ended in a GPU memory fault whose cause is not found; "
                          "kcg_gemm_f32 refuses operands of 2^31 elements and more until it is")
 def test_operands_beyond_two_to_the_31_elements(dev):
