@@ -20,18 +20,8 @@ SHAPES = [(1, 32, 2048, 128), (4, 32, 4096, 128), (2, 16, 8192, 128), (8, 32, 10
 
 
 def _time(fn, iters):
-    import torch
-    for _ in range(max(3, iters // 3)):
-        fn()
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    from kernelcodegen_amd.timing import time_launches
+    return time_launches(fn, iters)
 
 
 def main():

@@ -28,18 +28,8 @@ DIMS = [256, 512, 768, 1024, 1536, 2048, 3072, 4096, 5120, 6144, 7168, 8192, 921
 
 
 def _time(fn, iters):
-    import torch
-    for _ in range(max(3, iters // 4)):
-        fn()
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    from kernelcodegen_amd.timing import time_launches
+    return time_launches(fn, iters)
 
 
 def occupancy_percent(info):

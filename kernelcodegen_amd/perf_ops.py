@@ -25,18 +25,8 @@ PEAK_HBM_GBS = 8000.0
 
 
 def _time(fn, iters):
-    import torch
-    for _ in range(max(3, iters // 4)):
-        fn()
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    from kernelcodegen_amd.timing import time_launches
+    return time_launches(fn, iters)
 
 
 def main():
@@ -102,7 +92,7 @@ def main():
     print("| operator | ms | rate | bound | % of peak |")
     print("|---|---|---|---|---|")
     for r in rows:
-        print("| %s | %.4f | %s | %s | %.1f |" % r)
+        print(("| %s | %.4f | %s | %s | %.1f |" % r).replace("| nan |", "| - |"))
 
 
 if __name__ == "__main__":
