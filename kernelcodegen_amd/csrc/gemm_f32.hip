@@ -810,10 +810,12 @@ static GemmPlan default_plan(int64_t M, int64_t N) {
   const int64_t rows_of_tiles = (M + big.bm - 1) / big.bm;
   // Worth it only when a few tiles spill into one more round (tiles per CU = n + a small
   // fraction): workgroups of a launch run nearly in step, so those few hold the whole chip
-  // for a round; with a fraction around one half the measured loss is small (6144^3: 152).
+  // for a round.  With a fraction around one half the measured loss is nil at 6144^3 (152
+  // TFLOP/s either way) but grows with the size (14336^3: 145 as one launch, 150 cut).
   const int64_t tiles = rows_of_tiles * ((N + big.bn - 1) / big.bn);
   const int64_t spill = tiles % kNumCu;
-  if (tiles <= kNumCu || spill == 0 || spill * 20 > kNumCu * 7) return plan;
+  const int64_t max_spill = tiles >= 10 * kNumCu ? kNumCu * 11 / 20 : kNumCu * 7 / 20;
+  if (tiles <= kNumCu || spill == 0 || spill > max_spill) return plan;
   // the model prices the two launches as if the second waited for the last workgroup of the
   // first at full cost; measured, the cut does better than that by about 5 %
   constexpr double kSplitBias = 0.95;
