@@ -181,6 +181,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
   const int qrow = q0 + wave * 32 + r32;  // this lane's query
   const bool qvalid = qrow < S;
 
+  // the first K tile is requested before the Q rows so that both are in flight together
+  // (Ks is free: every wave passed the last barrier of the previous pass)
+  load_k(0);
+
   // ---- Q fragment: q[kk][j] = Q[qrow][8*kk + 4*half + j] * scale * log2(e) ----
   float4_t q[D / 8];
 #pragma unroll
@@ -204,7 +208,6 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const f
   const int kv_end = CAUSAL ? ((q0 + T::kBr) < S ? (q0 + T::kBr) : S) : S;
   const int n_tiles = (kv_end + BC - 1) / BC;
 
-  load_k(0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
