@@ -663,20 +663,30 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   // LDS may be handed to another workgroup once this one retires: drain the loads.
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), lgkmcnt/expcnt untouched
 
+  // A C that does not fit the 256 MiB last-level cache is streamed past it (non-temporal
+  // stores): with a short K the write of C is a large part of the run time.
+  auto store_c = [&](auto stream_c) {
 #pragma unroll
-  for (int i = 0; i < T::kTilesM; ++i) {
+    for (int i = 0; i < T::kTilesM; ++i) {
 #pragma unroll
-    for (int n = 0; n < T::kTilesN; ++n) {
-      const int col = n0 + wn * T::kWaveN + n * 32 + r32;
+      for (int n = 0; n < T::kTilesN; ++n) {
+        const int col = n0 + wn * T::kWaveN + n * 32 + r32;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm * T::kWaveM + i * 32 + 8 * (e / 4) + 4 * half + (e % 4);
-        float v = acc[i][n][e];
-        if (RELU) v = relu_maxf(v);
-        if (!RAGGED || (row < M && col < N)) C[static_cast<int64_t>(row) * N + col] = v;
+        for (int e = 0; e < 16; ++e) {
+          const int row = m0 + wm * T::kWaveM + i * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+          float v = acc[i][n][e];
+          if (RELU) v = relu_maxf(v);
+          if (!RAGGED || (row < M && col < N)) {
+            float *p = C + static_cast<int64_t>(row) * N + col;
+            if (decltype(stream_c)::value) __builtin_nontemporal_store(v, p);
+            else *p = v;
+          }
+        }
       }
     }
-  }
+  };
+  if (static_cast<int64_t>(M) * N * gridDim.y > (int64_t{48} << 20)) store_c(std::true_type{});
+  else store_c(std::false_type{});
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MIN_WAVES>
