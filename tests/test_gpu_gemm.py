@@ -223,6 +223,25 @@ def test_problems_cut_into_a_main_and_a_tail_launch(oracle, dev, shape, relu):
     assert max(rel_err(C, ref)) < TOL
 
 
+@pytest.mark.parametrize("shape", [(8192, 8192, 32), (8200, 6200, 36)])
+def test_output_larger_than_the_last_level_cache(dev, shape):
+    """A C of more than 48 Mi elements is written with non-temporal stores: every element must
+    still arrive (checked against a float64 product on row bands and on the whole-matrix sum)."""
+    import torch
+    from kernelcodegen_amd import ops
+    M, N, K = shape
+    A = torch.randn(M, K, device=dev)
+    B = torch.randn(K, N, device=dev)
+    C = torch.full((M, N), float("nan"), device=dev)
+    ops.matmul(A, B, relu=True, out=C)
+    assert not bool(torch.isnan(C).any())
+    for r0 in (0, M // 2 - 7, M - 300):
+        ref = torch.relu(A[r0:r0 + 300].double() @ B.double())
+        assert float((C[r0:r0 + 300].double() - ref).abs().max() / ref.abs().max()) < TOL
+    total = torch.relu(A.double() @ B.double()).sum()
+    assert abs(float(C.double().sum() - total)) / float(total) < 1e-6
+
+
 @pytest.mark.skip(reason="the one run of this case ended in a GPU memory fault whose cause is not found; "
                          "kcg_gemm_f32 refuses operands of 2^31 elements and more until it is")
 def test_operands_beyond_two_to_the_31_elements(dev):
