@@ -73,6 +73,14 @@ def main():
         info = lib.LaunchInfo()
         lib.check(L.kcg_gemm_f32_query(M, N, K, None, ctypes.byref(info)))
         mine = _time(lambda: ops.matmul(A, B, relu=args.relu, out=C), iters)
+        # the result of the timed launches against the library on three bands of rows
+        # (first, middle, last: the extremes of every operand's address range)
+        err = 0.0
+        for r0 in (0, max(0, M // 2 - 128), max(0, M - 256)):
+            ref = torch.matmul(A[r0:r0 + 256], B)
+            if args.relu:
+                ref = torch.relu(ref)
+            err = max(err, float((C[r0:r0 + 256] - ref).abs().max() / ref.abs().max()))
         nn = _time(lambda: torch.matmul(A, B, out=C), iters)
         # "TT": both operands transposed in memory, C^T = B^T . A^T
         tt = _time(lambda: torch.matmul(Bt, At, out=Ct), iters)
@@ -84,12 +92,13 @@ def main():
             mine, tf, 100 * tf / PEAK_FP32_TFLOPS))
         print("rocm-lib Latency(NN) = %g ms\nrocm-lib Ratio(NN) = %g%%\n" % (nn, 100 * nn / mine))
         print("rocm-lib Latency(TT) = %g ms\nrocm-lib Ratio(TT) = %g%%\n" % (tt, 100 * tt / mine), flush=True)
-        rows.append((M, N, K, mine, tf, 100 * tf / PEAK_FP32_TFLOPS, nn, flops / nn / 1e9))
+        print("max |C - library| / max |C| on sampled rows = %.2g\n" % err, flush=True)
+        rows.append((M, N, K, mine, tf, 100 * tf / PEAK_FP32_TFLOPS, nn, flops / nn / 1e9, err))
         del A, B, C, At, Bt, Ct
-    print("| M x N x K | kernel ms | TFLOP/s | % of 157.3 | library NN ms | library TFLOP/s |")
-    print("|---|---|---|---|---|---|")
+    print("| M x N x K | kernel ms | TFLOP/s | % of 157.3 | library NN ms | library TFLOP/s | max err vs library |")
+    print("|---|---|---|---|---|---|---|")
     for r in rows:
-        print("| %dx%dx%d | %.5g | %.2f | %.1f | %.5g | %.2f |" % r)
+        print("| %dx%dx%d | %.5g | %.2f | %.1f | %.5g | %.2f | %.1e |" % r)
 
 
 if __name__ == "__main__":
