@@ -804,7 +804,7 @@ static kcg_gemm_sched default_tile(int64_t M, int64_t N, int64_t batch, double *
 // in two along M: the first `main_rows` rows run on the 256 x 128 tile in whole rounds, the
 // rest on a small tile in a second launch on the same stream (rows of a row-major matrix are
 // contiguous, so both are ordinary matmuls on sub-matrices).  7168^3: 140 -> 149 TFLOP/s,
-// 9216^3: 144 -> 151, 3072^3: 125 -> 134.  main_rows == M: one launch.
+// 9216^3: 144 -> 152, 14336^3: 147 -> 153.  main_rows == M: one launch.
 struct GemmPlan {
   kcg_gemm_sched main;
   int64_t main_rows;
@@ -826,16 +826,13 @@ static GemmPlan default_plan(int64_t M, int64_t N) {
   const int64_t spill = tiles % kNumCu;
   const int64_t max_spill = tiles >= 10 * kNumCu ? kNumCu * 11 / 20 : kNumCu * 7 / 20;
   if (tiles <= kNumCu || spill == 0 || spill > max_spill) return plan;
-  // the model prices the two launches as if the second waited for the last workgroup of the
-  // first at full cost; measured, the cut does better than that by about 5 %
-  constexpr double kSplitBias = 0.95;
   double best = single;
   for (int64_t k = 1; k <= 8 && k < rows_of_tiles; ++k) {
     const int64_t m1 = (rows_of_tiles - k) * big.bm;
     const double c1 = tile_cost(big, m1, N, 1);
     double c2 = 0.0;
     const kcg_gemm_sched t = default_tile(M - m1, N, 1, &c2);
-    const double cost = (c1 + c2) * kSplitBias;
+    const double cost = c1 + c2;
     if (cost < best) {
       best = cost;
       plan.main = sched_of(big);

@@ -202,7 +202,7 @@ def test_shape_mismatch_raises(dev):
                    sched=dict(block_m=96))
 
 
-@pytest.mark.parametrize("shape", [(3072, 3072, 96), (4100, 4100, 64), (66000 // 8, 128 * 9, 40), (5120, 5120, 32)])
+@pytest.mark.parametrize("shape", [(7168, 7168, 32), (4100, 4100, 64), (66000 // 8, 128 * 9, 40), (5120, 5120, 32)])
 @pytest.mark.parametrize("relu", [False, True])
 def test_problems_cut_into_a_main_and_a_tail_launch(oracle, dev, shape, relu):
     """With no schedule given, a problem whose 256 x 128 tiles spill a little into one more
