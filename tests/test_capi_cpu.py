@@ -135,3 +135,33 @@ def test_tensors_of_two_to_the_31_elements_are_refused():
     assert L.kcg_batched_matmul_f32(fake, 0, fake, 1, fake, 64, 8192, 8192, 128, None) == unsupported
     assert L.kcg_fmha_f32(fake, fake, fake, fake, 64, 64, 4096, 128, 1.0, 0, None, None) == unsupported
     assert L.kcg_fmha_bf16(fake, fake, fake, fake, 1, 64, 64, 4096, 128, 1.0, 1, None, None) == unsupported
+
+
+def test_default_matmul_plans_cover_the_problem():
+    """Whatever the default chooser decides (one launch, or whole rounds of the large tile
+    plus a tail launch on a small tile), the launches it names cover every row of C exactly
+    once and the main launch is made of whole tile rows."""
+    import re
+    import numpy as np
+    L = lib.load()
+    info = lib.LaunchInfo()
+    rng = np.random.default_rng(7)
+    shapes = [(d, d) for d in range(1024, 16385, 1024)] + \
+             [(int(rng.integers(1, 40000)), int(rng.integers(1, 40000))) for _ in range(300)]
+    cut = 0
+    for M, N in shapes:
+        assert L.kcg_gemm_f32_query(M, N, 256, None, ctypes.byref(info)) == 0
+        name = info.kernel.decode()
+        m = re.fullmatch(r"gemm_f32_(\d+)x(\d+)x(\d+)_w\dx\d(?:_dl|_dl_ragged)?(?:\+(\d+)rows_(\d+)x(\d+)x(\d+))?", name)
+        assert m, name
+        bm, bn = int(m.group(1)), int(m.group(2))
+        tiles_n = -(-N // bn)
+        assert info.grid[0] % tiles_n == 0
+        main_rows = info.grid[0] // tiles_n * bm
+        if m.group(4) is None:
+            assert main_rows >= M and main_rows - M < bm, (M, N, name)
+        else:
+            cut += 1
+            assert (bm, bn) == (256, 128) and main_rows + int(m.group(4)) == M, (M, N, name)
+            assert int(m.group(4)) >= 1
+    assert cut > 10      # the sweep's odd multiples of 1024 at least
