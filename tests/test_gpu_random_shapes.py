@@ -92,3 +92,26 @@ def test_attention_random_shapes(oracle, dev):
             O = ops.fmha(_gpu(Q, dev), _gpu(K, dev), _gpu(V, dev), scale=scale, causal=causal,
                          sched=dict(br=br, bc=bc)).cpu().numpy()
             assert max(rel_err(O, ref)) < 1e-4, tag
+
+
+def test_batched_matmul_random_shapes(oracle, dev):
+    """All four layouts; extents around the tile edges, K around the slice depths, with and
+    without 16-byte aligned rows (aligned NN / NT run on the tiled kernel, the rest on the
+    generic one)."""
+    from kernelcodegen_amd import ops
+    rng = np.random.default_rng(20240602)
+    for case in range(40):
+        ta, tb = bool(case & 1) and case % 5 == 0, bool((case >> 1) & 1)
+        batch = tuple(int(x) for x in rng.integers(1, 4, size=int(rng.integers(0, 3))))
+        M, N = _extent(rng, 64, 300), _extent(rng, 64, 300)
+        K = _extent(rng, 16, 160)
+        if case % 3:
+            K = max(4, K // 4 * 4)          # 16-byte aligned rows of A (and of B^T)
+            if not tb:
+                N = max(4, N // 4 * 4)
+        A = inputs.normal(batch + ((K, M) if ta else (M, K)), 9700 + case, 0)
+        B = inputs.normal(batch + ((N, K) if tb else (K, N)), 9700 + case, 1)
+        ref = oracle.batched_matmul(A, ta, B, tb)
+        C = ops.batched_matmul(_gpu(A, dev), _gpu(B, dev), trans_a=ta, trans_b=tb).cpu().numpy()
+        assert C.shape == ref.shape
+        assert max(rel_err(C, ref)) < 1e-4, (case, batch, M, N, K, ta, tb)
