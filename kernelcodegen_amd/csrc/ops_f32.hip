@@ -158,8 +158,8 @@ __global__ __launch_bounds__(256) void softmax_f32_wave_rows_kernel(float *__res
   }
 }
 
-// Rows of up to 1024 * NV floats: one workgroup per row, the row in registers, maximum
-// and sum combined through LDS.
+// Rows of up to 1024 * NV floats (NV up to 32: 32768 floats, 128 registers): one workgroup
+// per row, the row in registers, maximum and sum combined through LDS.
 template <int NV, bool STREAM>
 __global__ __launch_bounds__(256) void softmax_f32_block_row_kernel(float *__restrict__ x, int n4) {
   __shared__ float red[8];
@@ -202,6 +202,46 @@ __global__ __launch_bounds__(256) void softmax_f32_block_row_kernel(float *__res
       if (STREAM) __builtin_nontemporal_store(r, p + c);
       else p[c] = r;
     }
+  }
+}
+
+// Rows of up to 256 * NV floats with no alignment to rely on (row length not a multiple of
+// 4): the same register-resident scheme with one float per access; consecutive lanes read
+// consecutive floats, so a wave still moves whole 256-byte segments.
+template <int NV>
+__global__ __launch_bounds__(256) void softmax_f32_block_row_scalar_kernel(float *__restrict__ x, int n) {
+  __shared__ float red[8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float *p = x + static_cast<int64_t>(blockIdx.x) * n;
+  constexpr float kLog2e = 1.4426950408889634f;
+  float v[NV];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = tid + 256 * i;
+    v[i] = c < n ? p[c] : -INFINITY;
+    m = fmaxf(m, v[i]);
+  }
+  m = wave_max(m);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float m_use = (m == -INFINITY) ? 0.0f : m;
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    v[i] = __builtin_amdgcn_exp2f((v[i] - m_use) * kLog2e);
+    sum += v[i];
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) red[4 + wave] = sum;
+  __syncthreads();
+  sum = (red[4] + red[5]) + (red[6] + red[7]);
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = tid + 256 * i;
+    if (c < n) p[c] = v[i] * inv;
   }
 }
 
@@ -256,7 +296,7 @@ int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream) {
   if (!x) return KCG_ERR_NULL_POINTER;
   if (rows <= 0 || n <= 0 || rows > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (n % 4 == 0 && n <= 8192 && kcg::aligned16(x)) {
+  if (n % 4 == 0 && n <= 32768 && kcg::aligned16(x)) {
     const int n4 = static_cast<int>(n / 4);
     // a tensor that does not fit the 256 MiB last-level cache is streamed past it
     const bool stream_past = rows * n * 4 > (int64_t{192} << 20);
@@ -276,9 +316,19 @@ int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream) {
     if (n4 <= 256) KCG_WAVE_ROWS(4);
     if (n4 <= 512) KCG_BLOCK_ROW(2);
     if (n4 <= 1024) KCG_BLOCK_ROW(4);
-    KCG_BLOCK_ROW(8);
+    if (n4 <= 2048) KCG_BLOCK_ROW(8);
+    if (n4 <= 4096) KCG_BLOCK_ROW(16);
+    KCG_BLOCK_ROW(32);
 #undef KCG_WAVE_ROWS
 #undef KCG_BLOCK_ROW
+  }
+  if (n <= 8192) {
+    const dim3 row_grid(static_cast<unsigned>(rows));
+    const int ni = static_cast<int>(n);
+    if (n <= 1024) return kcg::launch(kcg::softmax_f32_block_row_scalar_kernel<4>, row_grid, dim3(256), 0, s, x, ni);
+    if (n <= 2048) return kcg::launch(kcg::softmax_f32_block_row_scalar_kernel<8>, row_grid, dim3(256), 0, s, x, ni);
+    if (n <= 4096) return kcg::launch(kcg::softmax_f32_block_row_scalar_kernel<16>, row_grid, dim3(256), 0, s, x, ni);
+    return kcg::launch(kcg::softmax_f32_block_row_scalar_kernel<32>, row_grid, dim3(256), 0, s, x, ni);
   }
   return kcg::launch(kcg::softmax_f32_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, s, x, n);
 }

@@ -104,7 +104,8 @@ def test_batched_matmul_output_is_not_touched_outside_c(dev):
 
 @pytest.mark.parametrize("shape", [(4, 9, 33), (2, 2, 64, 64), (3, 1000), (5, 1), (2, 5000), (7, 4), (9, 256),
                                    (6, 260), (5, 1024), (3, 1028), (5, 2048), (3, 2052), (2, 4096), (3, 8192),
-                                   (2, 8196), (1, 3, 100)])
+                                   (2, 8196), (1, 3, 100), (3, 1001), (2, 2047), (3, 4099), (2, 8191), (2, 8193),
+                                   (2, 16384), (3, 12000), (2, 32768), (2, 32772), (1, 40000)])
 def test_softmax(oracle, dev, shape):
     from kernelcodegen_amd import ops
     x = inputs.normal(shape, 303, 0) * np.float32(2)
