@@ -87,7 +87,7 @@ int kcg_relu_f32(const float *x, float *y, int64_t n, void *stream) {
                        s, x, y, n4, n);
   } else {
     int64_t blocks = (n + threads - 1) / threads;
-    if (blocks > 256 * 32) blocks = 256 * 32;
+    if (blocks > 0x7fffffffLL) blocks = 0x7fffffffLL;
     return kcg::launch(kcg::relu_f32_scalar_kernel, dim3(static_cast<unsigned>(blocks)),
                        dim3(threads), 0, s, x, y, n);
   }
