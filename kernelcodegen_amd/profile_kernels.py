@@ -21,7 +21,11 @@ COPY_MIB = 256
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="gemm_cfg1",
-                    choices=["gemm_cfg0", "gemm_cfg1", "gemm_cfg2", "fmha_cfg3", "fmha_cfg4"])
+                    choices=["gemm_cfg0", "gemm_cfg1", "gemm_cfg2", "fmha_cfg3", "fmha_cfg4",
+                             "bmmnt_cfg3", "bmmnn_cfg3", "softmax_cfg3", "relu_1gib"],
+                    help="a BASELINE config of the fused kernels, or an un-fused operator at the "
+                         "configs[3] shape (bmmnt: Q.K^T, bmmnn: P.V, softmax: in place on the scores) "
+                         "/ ReLU on a 1 GiB tensor")
     ap.add_argument("--iters", type=int, default=200,
                     help="launches of the workload (the first tens run on a ramping clock)")
     args = ap.parse_args()
@@ -37,9 +41,25 @@ def main():
         dst.copy_(src)
     torch.cuda.synchronize()
 
-    kind, cfg = args.workload.split("_cfg")
-    c = inputs.config_inputs(int(cfg))
-    if kind == "gemm":
+    kind, _, cfg = args.workload.partition("_")
+    c = inputs.config_inputs(int(cfg[3:])) if cfg.startswith("cfg") else None
+    if kind == "relu":
+        X = torch.empty(16384, 16384, device=dev).normal_()
+        Y = torch.empty_like(X)
+        fn = lambda: ops.relu(X, out=Y)
+    elif kind in ("bmmnt", "bmmnn", "softmax"):
+        Q, K, V = (torch.from_numpy(c[k]).to(dev) for k in "QKV")
+        P = ops.batched_matmul(Q, K, trans_b=True)
+        O = torch.empty_like(Q)
+        if kind == "bmmnt":
+            fn = lambda: ops.batched_matmul(Q, K, trans_b=True, out=P)
+        elif kind == "bmmnn":
+            ops.softmax_(P.mul_(c["scale"]))
+            fn = lambda: ops.batched_matmul(P, V, out=O)
+        else:
+            P.mul_(c["scale"])
+            fn = lambda: ops.softmax_(P)
+    elif kind == "gemm":
         A = torch.from_numpy(c["A"]).to(dev)
         B = torch.from_numpy(c["B"]).to(dev)
         C = torch.empty((A.shape[0], B.shape[1]), dtype=torch.float32, device=dev)
