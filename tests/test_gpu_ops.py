@@ -198,9 +198,17 @@ def test_entry_points_can_be_captured_in_a_graph(dev):
     O = torch.empty_like(Q)
     Qb, Kb, Vb = Q.bfloat16(), K.bfloat16(), V.bfloat16()
     Ob = torch.empty_like(Qb)
+    # a size the default plan cuts into two launches, and a batched product and a softmax
+    A2 = torch.randn(5120, 32, device=dev)
+    B2 = torch.randn(32, 5120, device=dev)
+    C2 = torch.empty(5120, 5120, device=dev)
+    P = torch.empty(1, 2, 320, 320, device=dev)
 
     def launch_all():
         ops.matmul(A, B, relu=True, out=C)
+        ops.matmul(A2, B2, out=C2)
+        ops.batched_matmul(Q, K, trans_b=True, out=P)
+        ops.softmax_(P)
         ops.fmha(Q, K, V, scale=0.09, causal=True, out=O)
         ops.fmha(Qb, Kb, Vb, scale=0.09, causal=True, out=Ob)
 
@@ -211,18 +219,19 @@ def test_entry_points_can_be_captured_in_a_graph(dev):
         launch_all()
     for rep in range(3):
         A.normal_()
+        A2.normal_()
         Q.normal_()
         Qb.copy_(Q)
         launch_all()
         torch.cuda.synchronize()
-        want = (C.clone(), O.clone(), Ob.clone())
-        C.fill_(-1.0)
-        O.fill_(-1.0)
-        Ob.fill_(-1.0)
+        want = (C.clone(), O.clone(), Ob.clone(), C2.clone(), P.clone())
+        for t in (C, O, Ob, C2, P):
+            t.fill_(-1.0)
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(C, want[0]) and torch.equal(O, want[1]) and torch.equal(Ob, want[2]), rep
+        got = (C, O, Ob, C2, P)
+        assert all(torch.equal(g, w) for g, w in zip(got, want)), rep
 
 
 def test_concurrent_host_threads(oracle, dev):
