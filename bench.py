@@ -87,6 +87,8 @@ def main():
 
     import numpy as np
     import torch
+    import __graft_entry__
+    __graft_entry__.ensure_built()      # builds only if no library is there at all
     from kernelcodegen_amd import inputs, lib, ops
 
     if not torch.cuda.is_available():

@@ -13,6 +13,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+def pytest_sessionstart(session):
+    """A fresh checkout has no built library: build once (hipcc cross-compiles without a GPU).
+    A tree that holds a built library is used as it is."""
+    import __graft_entry__
+    __graft_entry__.ensure_built()
+
+
 def rel_err(x, y):
     """(max |x-y| / max(|y|, rms(y)),  max|x-y| / max|y|) -- both must pass a tolerance.
 
