@@ -72,6 +72,7 @@ int kcg_fmha_query(int dtype, int32_t B, int32_t H, int32_t S, int32_t D, int ca
 int kcg_relu_f32(const float *x, float *y, int64_t n, void *stream) {
   if (!x || !y) return KCG_ERR_NULL_POINTER;
   if (n <= 0) return KCG_ERR_BAD_SHAPE;
+  if (n > 0x7fffffffLL) return KCG_ERR_UNSUPPORTED_SHAPE;  // same limit as every entry point
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int threads = 256;
   if (kcg::aligned16(x) && kcg::aligned16(y)) {

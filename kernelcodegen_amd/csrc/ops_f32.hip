@@ -295,6 +295,7 @@ int kcg_batched_matmul_f32(const float *A, int transA, const float *B, int trans
 int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream) {
   if (!x) return KCG_ERR_NULL_POINTER;
   if (rows <= 0 || n <= 0 || rows > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
+  if (rows > 0x7fffffffLL / n) return KCG_ERR_UNSUPPORTED_SHAPE;  // same limit as every entry point
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (n % 4 == 0 && n <= 32768 && kcg::aligned16(x)) {
     const int n4 = static_cast<int>(n / 4);

@@ -135,6 +135,8 @@ def test_tensors_of_two_to_the_31_elements_are_refused():
     assert L.kcg_batched_matmul_f32(fake, 0, fake, 1, fake, 64, 8192, 8192, 128, None) == unsupported
     assert L.kcg_fmha_f32(fake, fake, fake, fake, 64, 64, 4096, 128, 1.0, 0, None, None) == unsupported
     assert L.kcg_fmha_bf16(fake, fake, fake, fake, 1, 64, 64, 4096, 128, 1.0, 1, None, None) == unsupported
+    assert L.kcg_relu_f32(fake, fake, 1 << 31, None) == unsupported
+    assert L.kcg_softmax_f32(fake, 1 << 20, 1 << 11, None) == unsupported
 
 
 def test_default_matmul_plans_cover_the_problem():
