@@ -18,7 +18,9 @@
  * src/Frontend/Operators.cc:271, include/KernelCodeGen.h:78-81) nothing here
  * aborts: every entry point returns a kcg_status.
  *
- * All entry points are thread-safe and hold no state between calls.
+ * All entry points are thread-safe and hold no state between calls.  A call may
+ * issue more than one kernel on the stream.  No tensor may have 2^31 elements
+ * or more (KCG_ERR_UNSUPPORTED_SHAPE).
  */
 #ifndef KCG_H
 #define KCG_H
