@@ -153,6 +153,27 @@ def test_unfused_graph_matches_fused_kernel(oracle, dev):
     assert max(rel_err(Of, O3)) < 1e-4
 
 
+def test_unfused_graph_at_full_size_matches_fused_kernel(oracle, dev):
+    """configs[3] (B=1, H=32, S=2048, D=128) as three kernels with the 512 MiB score tensor in
+    between, against the fused kernel on the whole output and against the oracle on sampled
+    query rows.  The scale goes into Q, so the graph itself is the reference's (scale 1)."""
+    from kernelcodegen_amd import ops
+    c = inputs.config_inputs(3)
+    Qs = (c["Q"] * np.float32(c["scale"])).astype(np.float32)
+    dQ, dK, dV = (_gpu(t, dev) for t in (Qs, c["K"], c["V"]))
+    P = ops.softmax_(ops.batched_matmul(dQ, dK, trans_b=True))
+    rows = P.sum(-1)
+    assert float((rows - 1).abs().max()) < 1e-4
+    O3 = ops.batched_matmul(P, dV)
+    Of = ops.fmha(dQ, dK, dV, scale=1.0, causal=False)
+    d = (O3 - Of).abs().max() / Of.abs().max()
+    assert float(d) < 1e-4
+    O3h = O3.cpu().numpy()
+    for r0, r1 in [(0, 8), (1023, 1031), (2040, 2048)]:
+        ref = oracle.fmha(Qs, c["K"], c["V"], scale=1.0, causal=False, stable=False, rows=(r0, r1))
+        assert max(rel_err(O3h[:, :, r0:r1], ref)) < 1e-4
+
+
 def test_launches_follow_the_callers_stream(oracle, dev):
     """Every entry point is asynchronous on the stream it is given: work queued on a side
     stream (default priority) is ordered after what that stream already holds and is not
