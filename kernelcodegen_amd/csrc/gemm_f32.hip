@@ -871,7 +871,10 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
   if (!s || (s->block_m == 0 && s->block_n == 0)) {
     const GemmPlan plan = default_plan(M, N);
     d = plan.main;
-    if (plan.main_rows < M) {
+    // a caller who fixes any tile field gets one launch with that field honoured
+    const bool free_choice = !s || (s->block_k == 0 && s->wave_m == 0 && s->wave_n == 0);
+    if (!free_choice) d = default_tile(M, N, 1);
+    if (free_choice && plan.main_rows < M) {
       // caller's remaining fields (GROUP_SIZE_M) apply to both launches
       kcg_gemm_sched t = plan.tail;
       if (s && s->group_m) d.group_m = t.group_m = s->group_m;
