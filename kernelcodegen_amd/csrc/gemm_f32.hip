@@ -665,6 +665,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 
   // A C that does not fit the 256 MiB last-level cache is streamed past it (non-temporal
   // stores): with a short K the write of C is a large part of the run time.
+  // Addresses are (uniform 64-bit tile origin) + (32-bit byte offset inside the tile): one
+  // 32-bit add per store instead of a 64-bit multiply-add -- VALU work that the short-K
+  // problems (attention scores: K = 128) would otherwise pay for in matrix time.  The
+  // offset stays below 2^32 because N < 2^22 on this path.
+  char *c_tile = reinterpret_cast<char *>(C + static_cast<int64_t>(m0) * N + n0);
+  const unsigned lane_off = (static_cast<unsigned>(wm * T::kWaveM + 4 * half) * static_cast<unsigned>(N) +
+                             static_cast<unsigned>(wn * T::kWaveN + r32)) * 4u;
+  const unsigned row_bytes = static_cast<unsigned>(N) * 4u;
   auto store_c = [&](auto stream_c) {
 #pragma unroll
     for (int i = 0; i < T::kTilesM; ++i) {
@@ -673,11 +681,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
         const int col = n0 + wn * T::kWaveN + n * 32 + r32;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const int row = m0 + wm * T::kWaveM + i * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+          const int local_row = i * 32 + 8 * (e / 4) + (e % 4);
+          const int row = m0 + wm * T::kWaveM + 4 * half + local_row;
           float v = acc[i][n][e];
           if (RELU) v = relu_maxf(v);
           if (!RAGGED || (row < M && col < N)) {
-            float *p = C + static_cast<int64_t>(row) * N + col;
+            float *p = reinterpret_cast<float *>(c_tile + (lane_off + static_cast<unsigned>(local_row) * row_bytes +
+                                                           static_cast<unsigned>(n * 32 * 4)));
             if (decltype(stream_c)::value) __builtin_nontemporal_store(v, p);
             else *p = v;
           }
@@ -710,7 +720,7 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
     info->waves_per_block = WAVES_M * WAVES_N;
     const char *kind = "";
     if constexpr (BK == 8 || BK == 16 || BK == 32) {
-      if ((full || ragged_dl) && K < (1 << 22) && N < (1 << 24)) {
+      if ((full || ragged_dl) && K < (1 << 22) && N < (1 << 22)) {
         info->lds_bytes = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>::kLdsBytes;
         kind = full ? "_dl" : "_dl_ragged";
       }
@@ -724,7 +734,7 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
   if constexpr (BK == 8 || BK == 16 || BK == 32) {
     using TD = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>;
     // the direct-load kernel addresses a slice with 32-bit byte offsets
-    if ((full || ragged_dl) && K < (1 << 22) && N < (1 << 24)) {
+    if ((full || ragged_dl) && K < (1 << 22) && N < (1 << 22)) {
       auto launch_dl = [&](auto kern) {
         if (!allow_lds(kern, TD::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
         return launch(kern, grid, block, TD::kLdsBytes, stream, A, B, C, static_cast<int>(M),
@@ -917,7 +927,7 @@ static int launch_bmm_dl(const float *A, const float *B, float *C, int64_t batch
                          int64_t K, bool trans_b, hipStream_t stream) {
   const int64_t tiles_m = (M + BM - 1) / BM;
   const int64_t tiles_n = (N + BN - 1) / BN;
-  if (tiles_m * tiles_n > 0x7fffffffLL || M > 0x7fffffffLL || N >= (1 << 24) || K >= (1 << 22) || batch > 65535)
+  if (tiles_m * tiles_n > 0x7fffffffLL || M > 0x7fffffffLL || N >= (1 << 22) || K >= (1 << 22) || batch > 65535)
     return KCG_ERR_UNSUPPORTED_SHAPE;
   if (K % 4 != 0 || K < BK || (!trans_b && N % 4 != 0) || !aligned16(A) || !aligned16(B))
     return KCG_ERR_UNSUPPORTED_SHAPE;
