@@ -46,6 +46,11 @@
 
 #include "kcg_common.h"
 
+#ifndef KCG_STAMP
+#define KCG_STAMP(id)
+#define KCG_TRACE_DECL
+#endif
+
 namespace kcg {
 
 typedef __bf16 bf16x8_v __attribute__((ext_vector_type(8)));
@@ -451,6 +456,511 @@ __global__ __launch_bounds__(64 * WAVES, (QT == 1 ? 2 : 1)) void fmha_bf16_kerne
   }
 }
 
+// ---------------------------------------------------------------------------
+// Ping-pong kernel: 8 waves, 256 query rows, two groups of four waves half a
+// tile apart.
+//
+// A wave64 VALU instruction issued beside the MFMAs of the *other* wave of its SIMD
+// costs that wave nothing (measured: the MFMA wave keeps one MFMA per 32 clocks), but
+// two waves that are in the same phase only contend: both wait for the matrix pipe,
+// then both for the vector ALU.  Waves w and w + 4 share a SIMD, so group 1 (waves
+// 4-7) runs one interval behind group 0 (waves 0-3), and every workgroup barrier ends
+// an interval:
+//
+//   interval     2t             2t+1           2t+2              2t+3
+//   group 0      PV(t-1), S(t)  softmax(t)     PV(t), S(t+1)     softmax(t+1)
+//   group 1      softmax(t-1)   PV(t-1), S(t)  softmax(t)        PV(t), S(t+1)
+//
+// In its matrix interval a wave is alone on the SIMD's matrix pipe, so nothing hides the
+// latency of its LDS operand reads but the wave itself: the 32 MFMAs of an interval take
+// their A operands from a queue of eight fragments that is refilled eight MFMAs ahead,
+// and the first eight are read at the end of the softmax interval, before the barrier.
+// Softmax arithmetic per tile and lane (32 scores): 16 v_max3 on the raw products, one
+// FMA + v_exp per score (exp2(s * c - m), c = scale * log2(e)), 16 v_cvt_pk, 32 v_add for
+// the row sum and a half-wave exchange -- about 640 clocks of vector issue against the
+// 1024 clocks of the partner wave's 32 MFMAs.  The row sum adds the fp32 exponentials:
+// v_dot2c_f32_bf16 on the packed pairs queues behind the partner wave's MFMAs (21 clocks
+// apiece instead of 4).  Q stays unscaled: scaling it once and rounding it to bf16 again
+// would save the FMAs but more than doubles the error against the fp32 evaluation.
+// K tiles live in a ring of 4 LDS buffers, V tiles in a ring of 5; the tile three steps
+// ahead is requested in the softmax interval (direct global -> LDS loads), when both
+// groups are done with the buffers it replaces.  The tiles of the second query block of
+// a causal pair follow those of the first in one stream, so the pipeline is filled once
+// per workgroup.
+template <int D>
+struct FmhaPpTile {
+  static constexpr int kWaves = 8;
+  static constexpr int kThreads = 64 * kWaves;
+  static constexpr int kBr = 32 * kWaves;
+  static constexpr int kBc = 64;
+  static constexpr int kCpr = D / 8;             // 16-byte chunks per row
+  static constexpr int kRowsPer256 = 16 / kCpr;  // rows that share one 256-byte bank window
+  static constexpr int kRpi = 64 / kCpr;         // rows filled by one wave-wide direct load
+  static constexpr int kIpw = kBc / kRpi / kWaves;  // direct loads per wave per K (or V) tile
+  static constexpr int kTile = kBc * D;          // elements per tile buffer
+  static constexpr int kAhead = 3;               // tiles requested ahead of the one in use
+  static constexpr int kRingK = 4;
+  static constexpr int kRingV = 5;
+  static constexpr int kLdsBytes = (kRingK + kRingV) * kTile * 2;
+  static constexpr int kDTiles = D / 32;
+  static constexpr int kDSteps = D / 16;
+  static constexpr int kPvMfmas = 4 * kDTiles;   // MFMAs of O += P.V per tile
+  static constexpr int kSMfmas = 2 * kDSteps;    // MFMAs of S = K.Q^T per tile
+  static constexpr int kQueue = 8;               // operand fragments read ahead of the MFMA that uses them
+  static_assert(D == 64 || D == 128, "head dim");
+  static_assert(kIpw >= 1 && kBc % (kWaves * kRpi) == 0, "tile extents");
+  static_assert(kPvMfmas >= kQueue && kSMfmas >= kQueue, "operand queue");
+  __host__ __device__ static constexpr int fk(int row) { return (row / kRowsPer256) % kCpr; }
+  __host__ __device__ static constexpr int fv(int row) { return 4 * ((row / kRowsPer256) & (kCpr / 4 - 1)); }
+};
+
+template <int D, bool CAUSAL, bool OUT_BF16>
+__global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    void *__restrict__ O, int S, int q_blocks, int q_items, float scale_log2e) {
+  using T = FmhaPpTile<D>;
+  constexpr int BC = T::kBc;
+  KCG_TRACE_DECL
+  extern __shared__ __align__(16) uint16_t lds16[];
+  uint16_t *Ks = lds16;                         // [kRingK][BC][D], chunk-swizzled
+  uint16_t *Vs = lds16 + T::kRingK * T::kTile;  // [kRingV][BC][D], chunk-swizzled
+
+  const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int bh = bid / q_items;
+  const int item = bid - bh * q_items;
+  const int hi_block = q_blocks - 1 - item;
+  const int npass = CAUSAL ? (hi_block != item ? 2 : 1) : 1;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int group = wave >> 2;
+  const int r32 = lane & 31;
+  const int half = lane >> 5;
+
+  const int64_t base = static_cast<int64_t>(bh) * S * D;
+  const uint16_t *Qb = Q + base;
+  const uint16_t *Kb = K + base;
+  const uint16_t *Vb = V + base;
+
+  // query block and tile count of a pass; the long block of a causal pair goes first
+  auto block_of = [&](int pass) { return CAUSAL ? (pass == 0 ? hi_block : item) : item; };
+  auto tiles_of = [&](int pass) {
+    const int q0 = block_of(pass) * T::kBr;
+    const int kv_end = CAUSAL ? ((q0 + T::kBr) < S ? (q0 + T::kBr) : S) : S;
+    return (kv_end + BC - 1) / BC;
+  };
+  const int n0 = tiles_of(0);
+  const int n1 = npass > 1 ? tiles_of(1) : 0;
+  const int n_all = n0 + n1;  // the K/V tiles of both passes form one stream
+
+  // ---- direct global -> LDS tile loads (same lane mapping as fmha_bf16_kernel) ----
+  const int ld_row0 = wave * T::kIpw * T::kRpi;
+  const int ld_lrow = lane / T::kCpr;
+  const int ld_pos = lane % T::kCpr;
+  unsigned goff_k[T::kIpw], goff_v[T::kIpw];
+#pragma unroll
+  for (int j = 0; j < T::kIpw; ++j) {
+    const int row = ld_row0 + j * T::kRpi + ld_lrow;
+    goff_k[j] = static_cast<unsigned>(row * D + (ld_pos ^ T::fk(row)) * 8) * 2u;
+    goff_v[j] = static_cast<unsigned>(row * D + (ld_pos ^ T::fv(row)) * 8) * 2u;
+  }
+  constexpr int kLoadsPerStep = 2 * T::kIpw;
+  const unsigned lds_k0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(Ks + ld_row0 * D));
+  const unsigned lds_v0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(Vs + ld_row0 * D));
+  int ld_ks = 0, ld_vs = 0;  // ring slots of the next tile of the stream
+  auto issue_next = [&](int jj) {
+    const int kv0 = (jj < n0 ? jj : jj - n0) * BC;
+    const char *kg = reinterpret_cast<const char *>(Kb + static_cast<int64_t>(kv0) * D);
+    const char *vg = reinterpret_cast<const char *>(Vb + static_cast<int64_t>(kv0) * D);
+    if (kv0 + BC <= S) {
+      // Issued from assembly (scalar base + 32-bit lane offset).  With the compiler's builtin
+      // every later LDS read is preceded by a wait for ALL outstanding direct loads
+      // (vmcnt(0)): it cannot tell which buffer they fill, and the tiles requested three
+      // steps ahead would be waited for at once.
+#pragma unroll
+      for (int j = 0; j < T::kIpw; ++j)
+        direct_load_16B(kg, goff_k[j], lds_k0 + static_cast<unsigned>((ld_ks * T::kTile + j * T::kRpi * D) * 2));
+#pragma unroll
+      for (int j = 0; j < T::kIpw; ++j)
+        direct_load_16B(vg, goff_v[j], lds_v0 + static_cast<unsigned>((ld_vs * T::kTile + j * T::kRpi * D) * 2));
+    } else {
+      // ragged last tile: rows at and beyond S are zero-filled, through registers
+      uint16_t *kl = Ks + ld_ks * T::kTile + ld_row0 * D;
+      uint16_t *vl = Vs + ld_vs * T::kTile + ld_row0 * D;
+#pragma unroll
+      for (int j = 0; j < T::kIpw; ++j) {
+        const int row = ld_row0 + j * T::kRpi + ld_lrow;
+        const bool ok = kv0 + row < S;
+        const u32x4_t z = {0u, 0u, 0u, 0u};
+        const u32x4_t kvq = ok ? *reinterpret_cast<const u32x4_t *>(kg + goff_k[j]) : z;
+        const u32x4_t vvq = ok ? *reinterpret_cast<const u32x4_t *>(vg + goff_v[j]) : z;
+        *reinterpret_cast<u32x4_t *>(kl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = kvq;
+        *reinterpret_cast<u32x4_t *>(vl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = vvq;
+      }
+      // (the compiler waits for these register loads with a vmcnt that ignores the direct
+      // loads above, i.e. a stricter one: counts are in issue order)
+    }
+    ld_ks = ld_ks == T::kRingK - 1 ? 0 : ld_ks + 1;
+    ld_vs = ld_vs == T::kRingV - 1 ? 0 : ld_vs + 1;
+  };
+  // Ends an interval (LDS reads and writes of this wave are complete first).
+  auto sync = [&]() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#ifndef KCG_FINE
+    KCG_STAMP(1);
+#endif
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#ifndef KCG_FINE
+    KCG_STAMP(2);
+#endif
+  };
+  // Waits until at most `steps` (0, 1 or 2) load steps of this wave are in flight.
+  auto wait_loads = [&](int steps) {
+    if (steps >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
+    else if (steps == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+
+  // ---- per-lane LDS read offsets (elements), swizzle folded in ----
+  const int k_row_off = r32 * D;
+  const int k_swz = T::fk(r32) ^ half;
+  const int l16 = lane & 15;
+  const int v_lrow = 4 * half + (l16 >> 2);
+  const int v_c0 = (2 * ((lane >> 4) & 1) + ((l16 & 3) >> 1)) ^ T::fv(v_lrow);
+  const int v_sub = 4 * (l16 & 1);
+  const int v_row_off = v_lrow * D + v_sub;
+
+  // ---- state of the current pass ----
+  bf16x8_v q[T::kDSteps];         // Q[wq0 + r32][16*s + 8*half .. +7]
+  float16_t acc_o[T::kDTiles];
+  float16_t s[2];                 // raw products of the tile at hand
+  unsigned p[2][8];               // bf16 pairs of P
+  bf16x8_v oq[T::kQueue];         // A-operand fragments read ahead (V^T, then K)
+  float m_ref = -INFINITY;        // reference maximum of the row (log2 units)
+  float l_run = 0.0f;             // this lane's share of the row sum
+  int wq0 = 0;
+
+  // Q rows of a pass, straight into the operand registers.  Issued from assembly and waited
+  // for by hand (q_ready): a load the compiler knows about, in a branch of the tile loop,
+  // makes it wait for every outstanding load (vmcnt(0)) before each later use of q, which
+  // would also drain the tile loads requested three steps ahead.  Rows at and beyond S read
+  // row S - 1 (their results are never stored).
+  auto load_q = [&](int pass) {
+    int row = block_of(pass) * T::kBr + wave * 32 + r32;
+    row = row < S ? row : S - 1;
+    const uint16_t *src = Qb + static_cast<int64_t>(row) * D + 8 * half;
+#pragma unroll
+    for (int ds = 0; ds < T::kDSteps; ++ds) {
+      u32x4_t v;
+      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(v) : "v"(src), "n"(32 * ds) : "memory");
+      q[ds] = __builtin_bit_cast(bf16x8_v, v);
+    }
+  };
+  // waits until at most `newer` vector memory operations issued after load_q are in flight
+  auto q_ready = [&](bool tile_loads_since) {
+    constexpr int kStores = 4 * T::kDTiles;  // stores of O issued since
+    if (tile_loads_since) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStores + kLoadsPerStep) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStores) : "memory");
+#pragma unroll
+    for (int ds = 0; ds < T::kDSteps; ++ds) asm volatile("" : "+v"(q[ds]));
+  };
+  auto start_pass = [&](int pass) {
+    wq0 = block_of(pass) * T::kBr + wave * 32;
+#pragma unroll
+    for (int i = 0; i < T::kDTiles; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc_o[i][e] = 0.0f;
+    m_ref = -INFINITY;
+    l_run = 0.0f;
+  };
+
+  // A operand of PV MFMA m (key block m / kDTiles of 16 keys, d tile m % kDTiles): V^T from
+  // the [key][d] tile with two transposing reads
+  auto read_v = [&](int vslot, int m) {
+    const int kb = m / T::kDTiles, i = m % T::kDTiles;
+    const uint16_t *vp = Vs + vslot * T::kTile + v_row_off + kb * 16 * D + ((4 * i) ^ v_c0) * 8;
+    const bf16x4_v lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((KCG_LDS_BF16X4 *)(vp));
+    const bf16x4_v hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((KCG_LDS_BF16X4 *)(vp + 8 * D));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  // A operand of S MFMA m (d step m / 2, key half m % 2): 8 bf16 of one K row
+  auto read_k = [&](int kslot, int m) {
+    const int ds = m / 2, kt = m % 2;
+    const uint16_t *kp = Ks + kslot * T::kTile + k_row_off + kt * 32 * D + ((2 * ds) ^ k_swz) * 8;
+    return __builtin_bit_cast(bf16x8_v, *reinterpret_cast<const u32x4_t *>(kp));
+  };
+  // B operand of PV MFMA m: the 16-key block m / kDTiles of P
+  auto p_block = [&](int m) {
+    const int kb = m / T::kDTiles;
+    const u32x4_t pw = {p[kb / 2][4 * (kb % 2)], p[kb / 2][4 * (kb % 2) + 1], p[kb / 2][4 * (kb % 2) + 2],
+                        p[kb / 2][4 * (kb % 2) + 3]};
+    return __builtin_bit_cast(bf16x8_v, pw);
+  };
+
+  // mask, reference maximum (lazy), P = exp2(s * c - m) packed to bf16, row sum
+  auto softmax = [&](int kv0) {
+    const int qrow = wq0 + r32;
+    if ((kv0 + BC > S) || (CAUSAL && (kv0 + BC - 1 > wq0))) {
+      // element (kt, e) is key kv0 + 4*half + off, off = 32*kt + 8*(e/4) + e%4; dead when off > lim
+      const int last = CAUSAL ? (qrow < S - 1 ? qrow : S - 1) : (S - 1);
+      const int lim = last - kv0 - 4 * half;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          if (32 * kt + 8 * (e / 4) + (e % 4) > lim) s[kt][e] = -INFINITY;
+    }
+    float mx0 = max3(s[0][0], s[0][1], s[0][2]), mx1 = max3(s[1][0], s[1][1], s[1][2]);
+#pragma unroll
+    for (int e = 3; e + 1 < 16; e += 2) {
+      mx0 = max3(mx0, s[0][e], s[0][e + 1]);
+      mx1 = max3(mx1, s[1][e], s[1][e + 1]);
+    }
+    // scale > 0: the maximum of the scaled scores is the scaled maximum (-inf stays -inf)
+#if defined(KCG_ABL) && KCG_ABL == 3
+    const float m_loc = 6.0f;
+#elif defined(KCG_ABL) && KCG_ABL == 8
+    const float m_loc = max3(mx0, mx1, fmaxf(s[0][15], s[1][15])) * scale_log2e;
+#else
+    const float m_loc = max_across_halves(max3(mx0, mx1, fmaxf(s[0][15], s[1][15]))) * scale_log2e;
+#endif
+    // per-row decision: a row's result never depends on what other rows do
+    if (m_loc > m_ref + kTau) {
+      const float alpha = __builtin_amdgcn_exp2f(m_ref - m_loc);  // m_ref = -inf -> 0
+      m_ref = m_loc;
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < T::kDTiles; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc_o[i][e] *= alpha;
+    }
+    const float neg_m = (m_ref == -INFINITY) ? 0.0f : -m_ref;
+    float ps[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+#if defined(KCG_ABL) && KCG_ABL == 4
+        const float p0 = (__builtin_fmaf(s[kt][2 * w], scale_log2e, neg_m));
+        const float p1 = (__builtin_fmaf(s[kt][2 * w + 1], scale_log2e, neg_m));
+#else
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * w], scale_log2e, neg_m));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * w + 1], scale_log2e, neg_m));
+#endif
+        p[kt][w] = pack_bf16(p0, p1);
+#if defined(KCG_ABL) && KCG_ABL == 12
+        ps[w & 3] += p0;
+        ps[(w + 2) & 3] += p1;
+#elif !defined(KCG_ABL) || KCG_ABL != 5
+        ps[w & 3] = add_bf16_pair(p[kt][w], ps[w & 3]);
+#endif
+      }
+    l_run += (ps[0] + ps[1]) + (ps[2] + ps[3]);
+  };
+
+  // normalise and store: lane holds O[qrow][32*i + 8*g + 4*half + 0..3]
+  auto store_o = [&]() {
+    const int qrow = wq0 + r32;
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float inv = 1.0f / l_tot;
+    if (qrow < S) {
+      const int64_t off = base + static_cast<int64_t>(qrow) * D + 4 * half;
+#pragma unroll
+      for (int i = 0; i < T::kDTiles; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const float v0 = acc_o[i][4 * g + 0] * inv;
+          const float v1 = acc_o[i][4 * g + 1] * inv;
+          const float v2 = acc_o[i][4 * g + 2] * inv;
+          const float v3 = acc_o[i][4 * g + 3] * inv;
+          if (OUT_BF16) {
+            u32x2_t w = {pack_bf16(v0, v1), pack_bf16(v2, v3)};
+            *reinterpret_cast<u32x2_t *>(static_cast<uint16_t *>(O) + off + 32 * i + 8 * g) = w;
+          } else {
+            float4_t w = {v0, v1, v2, v3};
+            *reinterpret_cast<float4_t *>(static_cast<float *>(O) + off + 32 * i + 8 * g) = w;
+          }
+        }
+    }
+  };
+
+#ifdef KCG_FINE
+  unsigned long long fine_ts[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+  unsigned long long f_prev = 0;
+#endif
+  // A wave whose last query precedes the tile has nothing to add (causal).
+  auto active = [&](int tile) { return !CAUSAL || (tile * BC <= wq0 + 31); };
+  const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  // the 2 * kDSteps MFMAs of S = K . Q^T from ring slot kslot; `primed`: the first kQueue
+  // fragments are already in the queue
+  auto s_phase = [&](int kslot, bool primed) {
+    if (!primed) {
+#pragma unroll
+      for (int m = 0; m < T::kQueue; ++m) oq[m] = read_k(kslot, m);
+    }
+#pragma unroll
+    for (int m = 0; m < T::kSMfmas; ++m) {
+      s[m % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oq[m % T::kQueue], q[m / 2], m < 2 ? zero16 : s[m % 2], 0, 0, 0);
+#if !defined(KCG_ABL) || KCG_ABL != 9
+      if (m + T::kQueue < T::kSMfmas) oq[m % T::kQueue] = read_k(kslot, m + T::kQueue);
+#endif
+      __builtin_amdgcn_sched_barrier(0);
+#ifdef KCG_FINE
+      if (m % 4 == 3) { fine_ts[4 + m / 4] = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); }
+#endif
+    }
+  };
+
+  // the 4 * kDTiles MFMAs of O += P . V; the queue holds the first kQueue fragments of V and
+  // is refilled kQueue MFMAs ahead, at the end with the first fragments of the next K tile
+  // (always: a branch here makes the compiler keep two copies of the accumulators and
+  // spill; when no S follows the fragments are simply not used)
+  auto pv_phase = [&](int vslot, int kslot) {
+#pragma unroll
+    for (int m = 0; m < T::kPvMfmas; ++m) {
+      acc_o[m % T::kDTiles] =
+          __builtin_amdgcn_mfma_f32_32x32x16_bf16(oq[m % T::kQueue], p_block(m), acc_o[m % T::kDTiles], 0, 0, 0);
+#if !defined(KCG_ABL) || KCG_ABL != 9
+      if (m + T::kQueue < T::kPvMfmas) oq[m % T::kQueue] = read_v(vslot, m + T::kQueue);
+      else oq[m % T::kQueue] = read_k(kslot, m + T::kQueue - T::kPvMfmas);
+#endif
+      __builtin_amdgcn_sched_barrier(0);
+#ifdef KCG_FINE
+      if (m % 4 == 3) { fine_ts[m / 4] = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); }
+#endif
+    }
+  };
+
+  // ---- prologue: the first tiles of the stream, then group 1 falls one interval behind ----
+  for (int jj = 0; jj < T::kAhead && jj < n_all; ++jj) issue_next(jj);
+  load_q(0);
+  start_pass(0);
+  wait_loads(0);
+#pragma unroll
+  for (int ds = 0; ds < T::kDSteps; ++ds) asm volatile("" : "+v"(q[ds]));
+  sync();
+  if (group == 1) sync();
+  int pass = 0;
+  int nt = n0;     // tiles of the current pass
+  int t = 0;       // tile (of the current pass) whose products are in s
+  int ks_next = 1; // ring slot of the K tile after that one
+  int vs_cur = 0;  // ring slot of its V tile
+  if (active(0)) s_phase(0, false);
+  sync();
+
+  for (int j = 0; j < n_all; ++j) {
+    // -- softmax interval, beside the other group's PV and S
+    const bool act = active(t);
+#ifdef KCG_FINE
+    const unsigned long long f_t0 = __builtin_readcyclecounter();
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+    // The last S of this pass is done: the Q registers are free for the next pass's rows,
+    // which then have this whole step to arrive (requested before this step's tile loads
+    // and before the stores of O, so that waiting for them waits for neither).
+    if (t + 1 == nt && pass + 1 < npass) load_q(pass + 1);
+    // requested first, so that their latency passes under the softmax arithmetic: the tile
+    // three steps ahead, and the first operands of PV(j) (V(j) was published one barrier ago)
+    const bool more = j + T::kAhead < n_all;
+#if !defined(KCG_ABL) || KCG_ABL != 2
+    if (more) issue_next(j + T::kAhead);
+#endif
+    if (act) {
+#pragma unroll
+      for (int m = 0; m < T::kQueue; ++m) oq[m] = read_v(vs_cur, m);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#ifdef KCG_FINE
+    const unsigned long long f_t1 = __builtin_readcyclecounter();
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+#if defined(KCG_ABL) && KCG_ABL == 11
+    if (act) {
+      // timing experiment: keep every MFMA alive with next to no vector work
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int w = 0; w < 8; ++w)
+          p[kt][w] = __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, s[kt][2 * w + 1]), __builtin_bit_cast(unsigned, s[kt][2 * w]), 0x07060302u);
+    }
+#elif !defined(KCG_ABL) || KCG_ABL != 1
+    if (act) softmax(t * BC);
+#endif
+    // Loads this wave may leave in flight: those of this step and of the step before.
+    // K(j+1) and V(j+1), requested two steps ago, are published by the coming barriers.
+    wait_loads((more ? 1 : 0) + (j + T::kAhead - 1 < n_all ? 1 : 0));
+#ifdef KCG_FINE
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const unsigned long long f_t2 = __builtin_readcyclecounter();
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+    sync();
+    // -- matrix interval: PV(j), then S(j+1); alone on the matrix pipe, ahead of the partner's VALU work
+#if !defined(KCG_ABL) || KCG_ABL != 7
+    __builtin_amdgcn_s_setprio(1);
+#endif
+#ifdef KCG_FINE
+    fine_ts[8] = __builtin_readcyclecounter();
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+    const bool last_of_pass = t + 1 == nt;
+    if (act) pv_phase(vs_cur, ks_next);
+    vs_cur = vs_cur == T::kRingV - 1 ? 0 : vs_cur + 1;
+    if (last_of_pass) {
+      store_o();
+      if (pass + 1 < npass) {
+        pass = 1;
+        nt = n1;
+        t = -1;
+        start_pass(1);
+        q_ready(more);
+      }
+    }
+    ++t;
+    if (j + 1 < n_all && active(t)) s_phase(ks_next, act);
+    ks_next = ks_next == T::kRingK - 1 ? 0 : ks_next + 1;
+#if !defined(KCG_ABL) || KCG_ABL != 7
+    __builtin_amdgcn_s_setprio(0);
+#endif
+    // group 1 ends the interval in which group 0 reads ahead into V(j+1): its own share of
+    // that tile and of K(j+2) (requested in its last softmax interval but one) must be in
+    if (group == 1) {
+      // (right after a pass switch the stores of O are the newest operations in flight:
+      // they need not be waited for)
+      if (t == 0 && j > 0 && more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * T::kDTiles + kLoadsPerStep) : "memory");
+      else wait_loads(more ? 1 : 0);
+    }
+#ifdef KCG_FINE
+    {
+      const unsigned long long t_a = __builtin_readcyclecounter();
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      asm volatile("s_nop 0\n\tv_mov_b32 %0, %0" : "+v"(l_run));
+      const unsigned long long t_b = __builtin_readcyclecounter();
+      __builtin_amdgcn_sched_barrier(0);
+      if (blockIdx.x == KCG_TRACE_WG && (threadIdx.x & 63) == 0 && j >= 8 && j < 12) {
+        long long *f = kcg_fine[threadIdx.x >> 6][j - 8];
+        f[0] = (long long)(f_t0 - f_prev);      // previous end-of-interval barrier wait (t6 of last iteration -> t0)
+        f[1] = (long long)(f_t1 - f_t0);        // softmax
+        f[2] = (long long)(f_t2 - f_t1);        // loads, prefetch, waits
+        f[3] = (long long)(fine_ts[8] - f_t2);  // barrier
+        f[4] = (long long)(fine_ts[7] - fine_ts[8]);  // 32 MFMAs issued
+        f[5] = (long long)(t_b - fine_ts[7]);   // tail
+        f[6] = (long long)(f_t2 & 0xffffff);           // absolute: arrival at the barrier that ends the softmax interval
+        f[7] = (long long)(fine_ts[8] & 0xffffff);     // absolute: first instruction after it
+        f[5] = (long long)(t_b & 0xffffff);            // absolute: arrival at the barrier that ends the matrix interval
+        f[0] = (long long)(f_t0 & 0xffffff);           // absolute: loop top (after the previous barrier)
+      }
+      f_prev = t_b;
+    }
+#endif
+    sync();
+  }
+  if (group == 0) sync();
+}
+
 template <int D, int BC, int QT, int WAVES, bool POS>
 static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O,
                             int o_dtype, int B, int H, int S, float scale, int causal,
@@ -491,6 +1001,37 @@ static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t
 #undef KCG_LAUNCH
 }
 
+template <int D>
+static int launch_fmha_bf16_pp(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O, int o_dtype,
+                               int B, int H, int S, float scale, int causal, hipStream_t stream,
+                               kcg_launch_info *info) {
+  using T = FmhaPpTile<D>;
+  const int64_t q_blocks = (static_cast<int64_t>(S) + T::kBr - 1) / T::kBr;
+  const int64_t q_items = causal ? (q_blocks + 1) / 2 : q_blocks;
+  const int64_t blocks = q_items * B * H;
+  if (blocks > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
+  if (info) {
+    info->grid[0] = static_cast<int>(blocks);
+    info->grid[1] = info->grid[2] = 1;
+    info->block[0] = T::kThreads;
+    info->block[1] = info->block[2] = 1;
+    info->lds_bytes = T::kLdsBytes;
+    info->waves_per_block = T::kWaves;
+    snprintf(info->kernel, sizeof info->kernel, "fmha_bf16_d%d_br%d_bc%d_pingpong%s", D, T::kBr, T::kBc,
+             causal ? "_causal_paired" : "");
+    return KCG_OK;
+  }
+  const float scale_log2e = scale * 1.4426950408889634f;
+  auto go = [&](auto kern) {
+    if (!allow_lds(kern, T::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
+    return launch(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads), T::kLdsBytes, stream, Q, K, V, O, S,
+                  static_cast<int>(q_blocks), static_cast<int>(q_items), scale_log2e);
+  };
+  const bool obf = o_dtype == KCG_BF16;
+  if (causal) return obf ? go(fmha_bf16_pp_kernel<D, true, true>) : go(fmha_bf16_pp_kernel<D, true, false>);
+  return obf ? go(fmha_bf16_pp_kernel<D, false, true>) : go(fmha_bf16_pp_kernel<D, false, false>);
+}
+
 int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O,
                        int o_dtype, int B, int H, int S, int D, float scale, int causal,
                        const kcg_fmha_sched *sched, hipStream_t stream, kcg_launch_info *info) {
@@ -518,8 +1059,7 @@ int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, 
     if (br == 128)                                                                                \
       return launch_fmha_bf16<D_, 64, 1, 4, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal,       \
                                                stream, info);                                     \
-    return launch_fmha_bf16<D_, 64, 1, 8, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, \
-                                             info);                                               \
+    return launch_fmha_bf16_pp<D_>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, info);      \
   }
   KCG_PICK(128)
   KCG_PICK(64)

@@ -61,26 +61,6 @@ struct FmhaF32Tile {
 // the accumulators are rescaled.
 constexpr float kTau = 8.0f;
 
-// v_max3_f32 without the canonicalising self-max the compiler puts in front of fmaxf on
-// MFMA results (NaN operands are ignored like in fmaxf; a NaN score still reaches the
-// output through its own exponential).
-__device__ __forceinline__ float max3(float a, float b, float c) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-#else
-  return fmaxf(fmaxf(a, b), c);
-#endif
-}
-
-// max over both halves of the wave for the same lane%32 (one v_permlane32_swap)
-__device__ __forceinline__ float max_across_halves(float x) {
-  const unsigned u = __builtin_bit_cast(unsigned, x);
-  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
-}
-
 template <int D, int BC, int WAVES, bool CAUSAL>
 __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const float *__restrict__ Q,
                                                           const float *__restrict__ K,

@@ -39,6 +39,33 @@ __device__ __forceinline__ float relu_maxf(float x) {
   return (x > 0.0f || x != x) ? x : 0.0f;
 }
 
+// v_max3_f32 without the canonicalising self-max the compiler puts in front of fmaxf on
+// MFMA results (NaN operands are ignored like in fmaxf; a NaN score still reaches the
+// output through its own exponential).
+__device__ __forceinline__ float max3(float a, float b, float c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+#else
+  return fmaxf(fmaxf(a, b), c);
+#endif
+}
+
+// max(x of lane l, x of lane l ^ 32): one v_permlane32_swap (the upper half of the first
+// register changes places with the lower half of the second) and one v_max.  Issued from
+// assembly: the compiler's builtin for this instruction hands back its first result
+// register for both results, which turns the maximum into "the lower half's value".
+__device__ __forceinline__ float max_across_halves(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+#else
+  return x;
+#endif
+}
+
 // One wave-wide direct load: lane l's 16 bytes at (uniform base + off) go to LDS byte
 // address lds_addr + 16 * l.  Issued from assembly so that the address is formed by the
 // instruction itself (scalar base + 32-bit lane offset); the intrinsic materialises a
