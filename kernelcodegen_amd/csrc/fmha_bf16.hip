@@ -7,6 +7,10 @@
 // Softmax -> BatchedMatmul(P, V) (test/test.cc:88-90), with the optional scale
 // and causal mask.
 //
+// Two kernels: fmha_bf16_kernel (described first; 4 waves, 128 query rows, also the general
+// softmax path for scale <= 0) and fmha_bf16_pp_kernel (8 waves, 256 query rows, its own
+// header further down), which long sequences that fill the chip take.
+//
 // Work split: WAVES (4 or 8) waves per workgroup, 32 query rows per wave
 // (Br = 128 or 256), K/V swept in tiles of BC = 64 rows.
 //
@@ -45,11 +49,6 @@
 #include <type_traits>
 
 #include "kcg_common.h"
-
-#ifndef KCG_STAMP
-#define KCG_STAMP(id)
-#define KCG_TRACE_DECL
-#endif
 
 namespace kcg {
 
@@ -458,7 +457,8 @@ __global__ __launch_bounds__(64 * WAVES, (QT == 1 ? 2 : 1)) void fmha_bf16_kerne
 
 // ---------------------------------------------------------------------------
 // Ping-pong kernel: 8 waves, 256 query rows, two groups of four waves half a
-// tile apart.
+// tile apart; one workgroup per CU walks its share of the launch as one stream
+// of K/V tiles.
 //
 // A wave64 VALU instruction issued beside the MFMAs of the *other* wave of its SIMD
 // costs that wave nothing (measured: the MFMA wave keeps one MFMA per 32 clocks), but
@@ -471,22 +471,29 @@ __global__ __launch_bounds__(64 * WAVES, (QT == 1 ? 2 : 1)) void fmha_bf16_kerne
 //   group 0      PV(t-1), S(t)  softmax(t)     PV(t), S(t+1)     softmax(t+1)
 //   group 1      softmax(t-1)   PV(t-1), S(t)  softmax(t)        PV(t), S(t+1)
 //
-// In its matrix interval a wave is alone on the SIMD's matrix pipe, so nothing hides the
-// latency of its LDS operand reads but the wave itself: the 32 MFMAs of an interval take
-// their A operands from a queue of eight fragments that is refilled eight MFMAs ahead,
-// and the first eight are read at the end of the softmax interval, before the barrier.
-// Softmax arithmetic per tile and lane (32 scores): 16 v_max3 on the raw products, one
-// FMA + v_exp per score (exp2(s * c - m), c = scale * log2(e)), 16 v_cvt_pk, 32 v_add for
-// the row sum and a half-wave exchange -- about 640 clocks of vector issue against the
-// 1024 clocks of the partner wave's 32 MFMAs.  The row sum adds the fp32 exponentials:
-// v_dot2c_f32_bf16 on the packed pairs queues behind the partner wave's MFMAs (21 clocks
-// apiece instead of 4).  Q stays unscaled: scaling it once and rounding it to bf16 again
-// would save the FMAs but more than doubles the error against the fp32 evaluation.
-// K tiles live in a ring of 4 LDS buffers, V tiles in a ring of 5; the tile three steps
-// ahead is requested in the softmax interval (direct global -> LDS loads), when both
-// groups are done with the buffers it replaces.  The tiles of the second query block of
-// a causal pair follow those of the first in one stream, so the pipeline is filled once
-// per workgroup.
+//  * In its matrix interval a wave is alone on the SIMD's matrix pipe, so nothing hides
+//    the latency of its LDS operand reads but the wave itself: the 32 MFMAs of an
+//    interval take their A operands from a queue of eight fragments that is refilled
+//    eight MFMAs ahead; the first eight are requested at the start of the softmax
+//    interval and arrive under its arithmetic.
+//  * The kernel runs at the socket's power limit, and what it buys there is fewer
+//    instructions per tile.  Softmax per tile and lane (32 scores): one FMA + v_exp per
+//    score (exp2(s * c - m), c = scale * log2(e)), 16 v_cvt_pk, 16 v_dot2c for the row sum
+//    and one half-wave exchange -- and no row maximum: the exponentials are taken
+//    against the reference the row already has, and only when the row sum shows that
+//    one of them exceeded 2^kTau (or on the row's first tile) is the maximum computed,
+//    the reference raised and the tile redone.  Q stays unscaled: scaling it once and
+//    rounding it to bf16 again would save the FMAs but more than doubles the error
+//    against the fp32 evaluation.
+//  * K tiles live in a ring of 4 LDS buffers, V tiles in a ring of 5; the tile three
+//    steps ahead is requested at the start of the softmax interval (direct global -> LDS
+//    loads issued from assembly), when both groups are done with the buffers it
+//    replaces.  All vector memory waits are counted by hand (wait_vm): the compiler
+//    would wait for every outstanding load before each LDS read or use of Q.
+//  * The K/V tiles of all query blocks a workgroup handles -- both blocks of a causal
+//    pair, then the next work item, possibly of another head -- follow each other in one
+//    stream, so the pipeline is filled once per workgroup; the Q rows of the next block
+//    are requested right after the last S of the current one.
 template <int D>
 struct FmhaPpTile {
   static constexpr int kWaves = 8;
@@ -517,19 +524,12 @@ struct FmhaPpTile {
 template <int D, bool CAUSAL, bool OUT_BF16>
 __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
-    void *__restrict__ O, int S, int q_blocks, int q_items, float scale_log2e) {
+    void *__restrict__ O, int S, int q_blocks, int q_items, int total_items, float scale_log2e) {
   using T = FmhaPpTile<D>;
   constexpr int BC = T::kBc;
-  KCG_TRACE_DECL
   extern __shared__ __align__(16) uint16_t lds16[];
   uint16_t *Ks = lds16;                         // [kRingK][BC][D], chunk-swizzled
   uint16_t *Vs = lds16 + T::kRingK * T::kTile;  // [kRingV][BC][D], chunk-swizzled
-
-  const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int bh = bid / q_items;
-  const int item = bid - bh * q_items;
-  const int hi_block = q_blocks - 1 - item;
-  const int npass = CAUSAL ? (hi_block != item ? 2 : 1) : 1;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -538,21 +538,44 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
   const int r32 = lane & 31;
   const int half = lane >> 5;
 
-  const int64_t base = static_cast<int64_t>(bh) * S * D;
-  const uint16_t *Qb = Q + base;
-  const uint16_t *Kb = K + base;
-  const uint16_t *Vb = V + base;
-
-  // query block and tile count of a pass; the long block of a causal pair goes first
-  auto block_of = [&](int pass) { return CAUSAL ? (pass == 0 ? hi_block : item) : item; };
-  auto tiles_of = [&](int pass) {
-    const int q0 = block_of(pass) * T::kBr;
-    const int kv_end = CAUSAL ? ((q0 + T::kBr) < S ? (q0 + T::kBr) : S) : S;
-    return (kv_end + BC - 1) / BC;
+  // Work items of this workgroup: an item is one (head, query block) or, causal, one (head,
+  // pair of query blocks (n-1-i, i)); a pass is one query block of an item.  The dispatcher
+  // deals workgroup w to XCD w % 8; every XCD owns a contiguous range of items (head-major,
+  // so the K/V of a head are fetched into one XCD's L2 only) and its workgroups take them
+  // round-robin: workgroups that run side by side then sweep the K/V of the same few heads
+  // at the same time and share each tile in that L2.
+  const int xcd = blockIdx.x % kNumXcd;
+  const int xcd_wgs = gridDim.x / kNumXcd + (xcd < static_cast<int>(gridDim.x % kNumXcd) ? 1 : 0);
+  // (a launch with one item per workgroup simply renumbers the workgroups XCD by XCD)
+  const bool one_each = static_cast<int>(gridDim.x) == total_items;
+  const int item_begin = one_each ? xcd_contiguous_id(blockIdx.x, gridDim.x)
+                                  : static_cast<int>(static_cast<int64_t>(xcd) * total_items / kNumXcd) + blockIdx.x / kNumXcd;
+  const int item_end = one_each ? item_begin + 1 : static_cast<int>(static_cast<int64_t>(xcd + 1) * total_items / kNumXcd);
+  const int item_step = xcd_wgs;
+  struct Pass {
+    int item, pass, npass, bh, block, nt;
   };
-  const int n0 = tiles_of(0);
-  const int n1 = npass > 1 ? tiles_of(1) : 0;
-  const int n_all = n0 + n1;  // the K/V tiles of both passes form one stream
+  auto describe = [&](Pass &c) {
+    c.bh = c.item / q_items;
+    const int it = c.item - c.bh * q_items;
+    const int hi = q_blocks - 1 - it;
+    c.npass = CAUSAL ? (hi != it ? 2 : 1) : 1;
+    c.block = CAUSAL ? (c.pass == 0 ? hi : it) : it;  // the long block of a causal pair goes first
+    const int q0 = c.block * T::kBr;
+    const int kv_end = CAUSAL ? ((q0 + T::kBr) < S ? (q0 + T::kBr) : S) : S;
+    c.nt = (kv_end + BC - 1) / BC;
+  };
+  // steps to the next pass; false when the workgroup's list is exhausted
+  auto next_pass = [&](Pass &c) {
+    if (++c.pass == c.npass) {
+      c.pass = 0;
+      c.item += item_step;
+      if (c.item >= item_end) return false;
+    }
+    describe(c);
+    return true;
+  };
+  if (item_begin >= item_end) return;  // (uniform: before any barrier)
 
   // ---- direct global -> LDS tile loads (same lane mapping as fmha_bf16_kernel) ----
   const int ld_row0 = wave * T::kIpw * T::kRpi;
@@ -566,13 +589,25 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
     goff_v[j] = static_cast<unsigned>(row * D + (ld_pos ^ T::fv(row)) * 8) * 2u;
   }
   constexpr int kLoadsPerStep = 2 * T::kIpw;
+  constexpr int kStores = 4 * T::kDTiles;  // vector stores of one pass's O rows
+  constexpr int kQLoads = T::kDSteps;      // vector loads of one pass's Q rows
   const unsigned lds_k0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(Ks + ld_row0 * D));
   const unsigned lds_v0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(Vs + ld_row0 * D));
-  int ld_ks = 0, ld_vs = 0;  // ring slots of the next tile of the stream
-  auto issue_next = [&](int jj) {
-    const int kv0 = (jj < n0 ? jj : jj - n0) * BC;
-    const char *kg = reinterpret_cast<const char *>(Kb + static_cast<int64_t>(kv0) * D);
-    const char *vg = reinterpret_cast<const char *>(Vb + static_cast<int64_t>(kv0) * D);
+  // The K/V tiles of all passes of all items form one stream; the load cursor runs kAhead
+  // tiles ahead of the tile being computed.
+  Pass lc = {item_begin, 0, 0, 0, 0, 0};
+  describe(lc);
+  int ld_tile = 0;        // next tile of lc to request
+  bool ld_valid = true;   // false once every tile of the list has been requested
+  int ld_ks = 0, ld_vs = 0;  // ring slots of that tile
+  // requests the next tile of the stream; returns the number of vector memory operations issued
+  auto issue_next = [&]() {
+    if (!ld_valid) return 0;
+    const int kv0 = ld_tile * BC;
+    const int64_t row0 = static_cast<int64_t>(lc.bh) * S + kv0;
+    const char *kg = reinterpret_cast<const char *>(K + row0 * D);
+    const char *vg = reinterpret_cast<const char *>(V + row0 * D);
+    int issued = kLoadsPerStep;
     if (kv0 + BC <= S) {
       // Issued from assembly (scalar base + 32-bit lane offset).  With the compiler's builtin
       // every later LDS read is preceded by a wait for ALL outstanding direct loads
@@ -585,7 +620,9 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
       for (int j = 0; j < T::kIpw; ++j)
         direct_load_16B(vg, goff_v[j], lds_v0 + static_cast<unsigned>((ld_vs * T::kTile + j * T::kRpi * D) * 2));
     } else {
-      // ragged last tile: rows at and beyond S are zero-filled, through registers
+      // ragged last tile: rows at and beyond S are zero-filled, through registers (the
+      // compiler waits for these loads itself, with a count that ignores the direct loads,
+      // i.e. a stricter one: counts are in issue order); nothing of it stays in flight
       uint16_t *kl = Ks + ld_ks * T::kTile + ld_row0 * D;
       uint16_t *vl = Vs + ld_vs * T::kTile + ld_row0 * D;
 #pragma unroll
@@ -598,30 +635,48 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
         *reinterpret_cast<u32x4_t *>(kl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = kvq;
         *reinterpret_cast<u32x4_t *>(vl + (j * T::kRpi + ld_lrow) * D + ld_pos * 8) = vvq;
       }
-      // (the compiler waits for these register loads with a vmcnt that ignores the direct
-      // loads above, i.e. a stricter one: counts are in issue order)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      issued = 0;
     }
     ld_ks = ld_ks == T::kRingK - 1 ? 0 : ld_ks + 1;
     ld_vs = ld_vs == T::kRingV - 1 ? 0 : ld_vs + 1;
+    if (++ld_tile == lc.nt) {
+      ld_tile = 0;
+      ld_valid = next_pass(lc);
+    }
+    return issued;
   };
   // Ends an interval (LDS reads and writes of this wave are complete first).
   auto sync = [&]() {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#ifndef KCG_FINE
-    KCG_STAMP(1);
-#endif
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-#ifndef KCG_FINE
-    KCG_STAMP(2);
-#endif
   };
-  // Waits until at most `steps` (0, 1 or 2) load steps of this wave are in flight.
-  auto wait_loads = [&](int steps) {
-    if (steps >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
-    else if (steps == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // Waits until at most n (even, <= 62) of this wave's vector memory operations are in flight.
+  auto wait_vm = [&](int n) {
+    // the two counts that occur in nearly every step come first
+    if (n == 2 * kLoadsPerStep) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
+      return;
+    }
+    if (n == kLoadsPerStep) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
+      return;
+    }
+    switch (n >> 1) {
+#define KCG_VM_CASE(h) \
+  case h: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (h)) : "memory"); break;
+      KCG_VM_CASE(1) KCG_VM_CASE(2) KCG_VM_CASE(3) KCG_VM_CASE(4) KCG_VM_CASE(5) KCG_VM_CASE(6) KCG_VM_CASE(7)
+      KCG_VM_CASE(8) KCG_VM_CASE(9) KCG_VM_CASE(10) KCG_VM_CASE(11) KCG_VM_CASE(12) KCG_VM_CASE(13)
+      KCG_VM_CASE(14) KCG_VM_CASE(15) KCG_VM_CASE(16) KCG_VM_CASE(17) KCG_VM_CASE(18) KCG_VM_CASE(19)
+      KCG_VM_CASE(20) KCG_VM_CASE(21) KCG_VM_CASE(22) KCG_VM_CASE(23) KCG_VM_CASE(24) KCG_VM_CASE(25)
+      KCG_VM_CASE(26) KCG_VM_CASE(27) KCG_VM_CASE(28) KCG_VM_CASE(29) KCG_VM_CASE(30) KCG_VM_CASE(31)
+#undef KCG_VM_CASE
+      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
   };
+  static_assert(kLoadsPerStep % 2 == 0 && kStores % 2 == 0 && kQLoads % 2 == 0, "wait_vm takes even counts");
+  static_assert(2 * kLoadsPerStep + 2 * (kStores + kQLoads) <= 62, "vmcnt range");
 
   // ---- per-lane LDS read offsets (elements), swizzle folded in ----
   const int k_row_off = r32 * D;
@@ -633,6 +688,8 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
   const int v_row_off = v_lrow * D + v_sub;
 
   // ---- state of the current pass ----
+  Pass cc = {item_begin, 0, 0, 0, 0, 0};
+  describe(cc);
   bf16x8_v q[T::kDSteps];         // Q[wq0 + r32][16*s + 8*half .. +7]
   float16_t acc_o[T::kDTiles];
   float16_t s[2];                 // raw products of the tile at hand
@@ -643,31 +700,26 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
   int wq0 = 0;
 
   // Q rows of a pass, straight into the operand registers.  Issued from assembly and waited
-  // for by hand (q_ready): a load the compiler knows about, in a branch of the tile loop,
-  // makes it wait for every outstanding load (vmcnt(0)) before each later use of q, which
-  // would also drain the tile loads requested three steps ahead.  Rows at and beyond S read
-  // row S - 1 (their results are never stored).
-  auto load_q = [&](int pass) {
-    int row = block_of(pass) * T::kBr + wave * 32 + r32;
+  // for by hand: a load the compiler knows about, in a branch of the tile loop, makes it
+  // wait for every outstanding load (vmcnt(0)) before each later use of q, which would also
+  // drain the tile loads requested three steps ahead.  Rows at and beyond S read row S - 1
+  // (their results are never stored).
+  auto load_q = [&](const Pass &c) {
+    int row = c.block * T::kBr + wave * 32 + r32;
     row = row < S ? row : S - 1;
-    const uint16_t *src = Qb + static_cast<int64_t>(row) * D + 8 * half;
+    const uint16_t *src = Q + (static_cast<int64_t>(c.bh) * S + row) * D + 8 * half;
+    // (in-out operands: the new rows land in the very registers that hold the old ones, so
+    // that no register copy can be placed between the request and the wait)
 #pragma unroll
-    for (int ds = 0; ds < T::kDSteps; ++ds) {
-      u32x4_t v;
-      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(v) : "v"(src), "n"(32 * ds) : "memory");
-      q[ds] = __builtin_bit_cast(bf16x8_v, v);
-    }
+    for (int ds = 0; ds < T::kDSteps; ++ds)
+      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "+v"(q[ds]) : "v"(src), "n"(32 * ds) : "memory");
   };
-  // waits until at most `newer` vector memory operations issued after load_q are in flight
-  auto q_ready = [&](bool tile_loads_since) {
-    constexpr int kStores = 4 * T::kDTiles;  // stores of O issued since
-    if (tile_loads_since) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStores + kLoadsPerStep) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStores) : "memory");
+  auto q_arrived = [&]() {
 #pragma unroll
     for (int ds = 0; ds < T::kDSteps; ++ds) asm volatile("" : "+v"(q[ds]));
   };
-  auto start_pass = [&](int pass) {
-    wq0 = block_of(pass) * T::kBr + wave * 32;
+  auto start_pass = [&]() {
+    wq0 = cc.block * T::kBr + wave * 32;
 #pragma unroll
     for (int i = 0; i < T::kDTiles; ++i)
 #pragma unroll
@@ -699,7 +751,7 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
     return __builtin_bit_cast(bf16x8_v, pw);
   };
 
-  // mask, reference maximum (lazy), P = exp2(s * c - m) packed to bf16, row sum
+  // mask, P = exp2(s * c - m) packed to bf16, row sum; reference maximum only when needed
   auto softmax = [&](int kv0) {
     const int qrow = wq0 + r32;
     if ((kv0 + BC > S) || (CAUSAL && (kv0 + BC - 1 > wq0))) {
@@ -712,52 +764,48 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
         for (int e = 0; e < 16; ++e)
           if (32 * kt + 8 * (e / 4) + (e % 4) > lim) s[kt][e] = -INFINITY;
     }
-    float mx0 = max3(s[0][0], s[0][1], s[0][2]), mx1 = max3(s[1][0], s[1][1], s[1][2]);
+    // P = exp2(s * c - m) as bf16 pairs; returns this lane's share of the row sum
+    auto exp_tile = [&](float neg_m) {
+      float ps[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int e = 3; e + 1 < 16; e += 2) {
-      mx0 = max3(mx0, s[0][e], s[0][e + 1]);
-      mx1 = max3(mx1, s[1][e], s[1][e + 1]);
-    }
-    // scale > 0: the maximum of the scaled scores is the scaled maximum (-inf stays -inf)
-#if defined(KCG_ABL) && KCG_ABL == 3
-    const float m_loc = 6.0f;
-#elif defined(KCG_ABL) && KCG_ABL == 8
-    const float m_loc = max3(mx0, mx1, fmaxf(s[0][15], s[1][15])) * scale_log2e;
-#else
-    const float m_loc = max_across_halves(max3(mx0, mx1, fmaxf(s[0][15], s[1][15]))) * scale_log2e;
-#endif
-    // per-row decision: a row's result never depends on what other rows do
-    if (m_loc > m_ref + kTau) {
-      const float alpha = __builtin_amdgcn_exp2f(m_ref - m_loc);  // m_ref = -inf -> 0
-      m_ref = m_loc;
-      l_run *= alpha;
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int i = 0; i < T::kDTiles; ++i)
+        for (int w = 0; w < 8; ++w) {
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * w], scale_log2e, neg_m));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * w + 1], scale_log2e, neg_m));
+          p[kt][w] = pack_bf16(p0, p1);
+          ps[w & 3] = add_bf16_pair(p[kt][w], ps[w & 3]);
+        }
+      return (ps[0] + ps[1]) + (ps[2] + ps[3]);
+    };
+    // Fast path: no row maximum at all.  The exponentials are taken against the reference
+    // the row already has; if one of them came out larger than 2^kTau the sum shows it
+    // (every term is >= 0), and only then -- and on a row's first tile -- is the maximum
+    // computed, the reference raised and the tile's exponentials taken again.  Both halves
+    // of the wave see the same sum and the same reference, so they decide alike.
+    float psum = exp_tile((m_ref == -INFINITY) ? 0.0f : -m_ref);
+    const float big = max_across_halves(psum);
+    if (m_ref == -INFINITY || big > 256.0f /* 2^kTau */) {
+      float mx0 = max3(s[0][0], s[0][1], s[0][2]), mx1 = max3(s[1][0], s[1][1], s[1][2]);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc_o[i][e] *= alpha;
-    }
-    const float neg_m = (m_ref == -INFINITY) ? 0.0f : -m_ref;
-    float ps[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int w = 0; w < 8; ++w) {
-#if defined(KCG_ABL) && KCG_ABL == 4
-        const float p0 = (__builtin_fmaf(s[kt][2 * w], scale_log2e, neg_m));
-        const float p1 = (__builtin_fmaf(s[kt][2 * w + 1], scale_log2e, neg_m));
-#else
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * w], scale_log2e, neg_m));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][2 * w + 1], scale_log2e, neg_m));
-#endif
-        p[kt][w] = pack_bf16(p0, p1);
-#if defined(KCG_ABL) && KCG_ABL == 12
-        ps[w & 3] += p0;
-        ps[(w + 2) & 3] += p1;
-#elif !defined(KCG_ABL) || KCG_ABL != 5
-        ps[w & 3] = add_bf16_pair(p[kt][w], ps[w & 3]);
-#endif
+      for (int e = 3; e + 1 < 16; e += 2) {
+        mx0 = max3(mx0, s[0][e], s[0][e + 1]);
+        mx1 = max3(mx1, s[1][e], s[1][e + 1]);
       }
-    l_run += (ps[0] + ps[1]) + (ps[2] + ps[3]);
+      // scale > 0: the maximum of the scaled scores is the scaled maximum (-inf stays -inf)
+      const float m_loc = max_across_halves(max3(mx0, mx1, fmaxf(s[0][15], s[1][15]))) * scale_log2e;
+      if (m_loc > m_ref) {
+        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_loc);  // m_ref = -inf -> 0
+        m_ref = m_loc;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < T::kDTiles; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc_o[i][e] *= alpha;
+      }
+      psum = exp_tile((m_ref == -INFINITY) ? 0.0f : -m_ref);
+    }
+    l_run += psum;
   };
 
   // normalise and store: lane holds O[qrow][32*i + 8*g + 4*half + 0..3]
@@ -766,7 +814,7 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv = 1.0f / l_tot;
     if (qrow < S) {
-      const int64_t off = base + static_cast<int64_t>(qrow) * D + 4 * half;
+      const int64_t off = (static_cast<int64_t>(cc.bh) * S + qrow) * D + 4 * half;
 #pragma unroll
       for (int i = 0; i < T::kDTiles; ++i)
 #pragma unroll
@@ -785,11 +833,11 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
         }
     }
   };
+  // Stores a wave is known to issue for a pass: all of them when every row is inside the
+  // sequence; a wave with rows beyond S may skip the instructions altogether, so it counts
+  // none (the hand-counted waits then wait for more than they need, never for less).
+  auto stores_of_pass = [&]() { return wq0 + 32 <= S ? kStores : 0; };
 
-#ifdef KCG_FINE
-  unsigned long long fine_ts[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
-  unsigned long long f_prev = 0;
-#endif
   // A wave whose last query precedes the tile has nothing to add (causal).
   auto active = [&](int tile) { return !CAUSAL || (tile * BC <= wq0 + 31); };
   const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -803,16 +851,10 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
 #pragma unroll
     for (int m = 0; m < T::kSMfmas; ++m) {
       s[m % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oq[m % T::kQueue], q[m / 2], m < 2 ? zero16 : s[m % 2], 0, 0, 0);
-#if !defined(KCG_ABL) || KCG_ABL != 9
       if (m + T::kQueue < T::kSMfmas) oq[m % T::kQueue] = read_k(kslot, m + T::kQueue);
-#endif
       __builtin_amdgcn_sched_barrier(0);
-#ifdef KCG_FINE
-      if (m % 4 == 3) { fine_ts[4 + m / 4] = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); }
-#endif
     }
   };
-
   // the 4 * kDTiles MFMAs of O += P . V; the queue holds the first kQueue fragments of V and
   // is refilled kQueue MFMAs ahead, at the end with the first fragments of the next K tile
   // (always: a branch here makes the compiler keep two copies of the accumulators and
@@ -822,141 +864,98 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
     for (int m = 0; m < T::kPvMfmas; ++m) {
       acc_o[m % T::kDTiles] =
           __builtin_amdgcn_mfma_f32_32x32x16_bf16(oq[m % T::kQueue], p_block(m), acc_o[m % T::kDTiles], 0, 0, 0);
-#if !defined(KCG_ABL) || KCG_ABL != 9
       if (m + T::kQueue < T::kPvMfmas) oq[m % T::kQueue] = read_v(vslot, m + T::kQueue);
       else oq[m % T::kQueue] = read_k(kslot, m + T::kQueue - T::kPvMfmas);
-#endif
       __builtin_amdgcn_sched_barrier(0);
-#ifdef KCG_FINE
-      if (m % 4 == 3) { fine_ts[m / 4] = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); }
-#endif
     }
   };
 
+  // Vector memory operations of this wave, newest first, as far back as the waits look:
+  //   d_cur / d_prev: tile loads of this step / the step before (softmax interval)
+  //   x_cur / x_prev / x_prev2: O stores and Q loads of this step's matrix interval / the
+  //   two steps before
+  int d_cur = 0, d_prev = 0, x_cur = 0, x_prev = 0, x_prev2 = 0;
+  // The pass after the current one, if any (its Q rows are requested as soon as the last S
+  // of the current pass has been issued).
+  Pass np = cc;
+  bool np_valid = next_pass(np);
+
   // ---- prologue: the first tiles of the stream, then group 1 falls one interval behind ----
-  for (int jj = 0; jj < T::kAhead && jj < n_all; ++jj) issue_next(jj);
-  load_q(0);
-  start_pass(0);
-  wait_loads(0);
-#pragma unroll
-  for (int ds = 0; ds < T::kDSteps; ++ds) asm volatile("" : "+v"(q[ds]));
+  for (int jj = 0; jj < T::kAhead; ++jj) issue_next();
+  load_q(cc);
+  start_pass();
+  wait_vm(0);
+  q_arrived();
   sync();
   if (group == 1) sync();
-  int pass = 0;
-  int nt = n0;     // tiles of the current pass
   int t = 0;       // tile (of the current pass) whose products are in s
   int ks_next = 1; // ring slot of the K tile after that one
   int vs_cur = 0;  // ring slot of its V tile
   if (active(0)) s_phase(0, false);
+  if (cc.nt == 1 && np_valid) {
+    load_q(np);
+    x_cur = kQLoads;
+  }
   sync();
+  x_prev = x_cur;
+  x_cur = 0;
 
-  for (int j = 0; j < n_all; ++j) {
+  for (bool running = true; running;) {
     // -- softmax interval, beside the other group's PV and S
     const bool act = active(t);
-#ifdef KCG_FINE
-    const unsigned long long f_t0 = __builtin_readcyclecounter();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
-    // The last S of this pass is done: the Q registers are free for the next pass's rows,
-    // which then have this whole step to arrive (requested before this step's tile loads
-    // and before the stores of O, so that waiting for them waits for neither).
-    if (t + 1 == nt && pass + 1 < npass) load_q(pass + 1);
     // requested first, so that their latency passes under the softmax arithmetic: the tile
-    // three steps ahead, and the first operands of PV(j) (V(j) was published one barrier ago)
-    const bool more = j + T::kAhead < n_all;
-#if !defined(KCG_ABL) || KCG_ABL != 2
-    if (more) issue_next(j + T::kAhead);
-#endif
+    // three steps ahead, and the first operands of PV (this V tile was published one barrier ago)
+    d_cur = issue_next();
     if (act) {
 #pragma unroll
       for (int m = 0; m < T::kQueue; ++m) oq[m] = read_v(vs_cur, m);
     }
     __builtin_amdgcn_sched_barrier(0);
-#ifdef KCG_FINE
-    const unsigned long long f_t1 = __builtin_readcyclecounter();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
-#if defined(KCG_ABL) && KCG_ABL == 11
-    if (act) {
-      // timing experiment: keep every MFMA alive with next to no vector work
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int w = 0; w < 8; ++w)
-          p[kt][w] = __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, s[kt][2 * w + 1]), __builtin_bit_cast(unsigned, s[kt][2 * w]), 0x07060302u);
-    }
-#elif !defined(KCG_ABL) || KCG_ABL != 1
     if (act) softmax(t * BC);
-#endif
-    // Loads this wave may leave in flight: those of this step and of the step before.
-    // K(j+1) and V(j+1), requested two steps ago, are published by the coming barriers.
-    wait_loads((more ? 1 : 0) + (j + T::kAhead - 1 < n_all ? 1 : 0));
-#ifdef KCG_FINE
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    const unsigned long long f_t2 = __builtin_readcyclecounter();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
+    // Still allowed in flight: the tile loads of this step and of the step before, and
+    // whatever the two last matrix intervals issued after the older of them.  The K and V
+    // tiles requested two steps ago are published by the coming barriers.
+    wait_vm(d_cur + d_prev + x_prev + x_prev2);
     sync();
-    // -- matrix interval: PV(j), then S(j+1); alone on the matrix pipe, ahead of the partner's VALU work
-#if !defined(KCG_ABL) || KCG_ABL != 7
+    // -- matrix interval: PV, then S of the next tile; alone on the matrix pipe
     __builtin_amdgcn_s_setprio(1);
-#endif
-#ifdef KCG_FINE
-    fine_ts[8] = __builtin_readcyclecounter();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
-    const bool last_of_pass = t + 1 == nt;
+    const bool last_of_pass = t + 1 == cc.nt;
+    const bool has_next = !last_of_pass || np_valid;
     if (act) pv_phase(vs_cur, ks_next);
     vs_cur = vs_cur == T::kRingV - 1 ? 0 : vs_cur + 1;
     if (last_of_pass) {
       store_o();
-      if (pass + 1 < npass) {
-        pass = 1;
-        nt = n1;
+      const int stores = stores_of_pass();
+      x_cur += stores;
+      if (np_valid) {
+        // the Q rows were requested one step ago, after the last S of the pass that ends
+        // here; newer than them: this step's tile loads and the stores just issued
+        cc = np;
+        np_valid = next_pass(np);
         t = -1;
-        start_pass(1);
-        q_ready(more);
+        start_pass();
+        wait_vm(d_cur + stores);
+        q_arrived();
       }
     }
     ++t;
-    if (j + 1 < n_all && active(t)) s_phase(ks_next, act);
+    if (has_next && active(t)) s_phase(ks_next, act);
+    if (has_next && t + 1 == cc.nt && np_valid) {
+      load_q(np);  // this was the pass's last S: the Q registers are free
+      x_cur += kQLoads;
+    }
     ks_next = ks_next == T::kRingK - 1 ? 0 : ks_next + 1;
-#if !defined(KCG_ABL) || KCG_ABL != 7
     __builtin_amdgcn_s_setprio(0);
-#endif
-    // group 1 ends the interval in which group 0 reads ahead into V(j+1): its own share of
-    // that tile and of K(j+2) (requested in its last softmax interval but one) must be in
-    if (group == 1) {
-      // (right after a pass switch the stores of O are the newest operations in flight:
-      // they need not be waited for)
-      if (t == 0 && j > 0 && more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * T::kDTiles + kLoadsPerStep) : "memory");
-      else wait_loads(more ? 1 : 0);
-    }
-#ifdef KCG_FINE
-    {
-      const unsigned long long t_a = __builtin_readcyclecounter();
-      __builtin_amdgcn_sched_barrier(0);
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      asm volatile("s_nop 0\n\tv_mov_b32 %0, %0" : "+v"(l_run));
-      const unsigned long long t_b = __builtin_readcyclecounter();
-      __builtin_amdgcn_sched_barrier(0);
-      if (blockIdx.x == KCG_TRACE_WG && (threadIdx.x & 63) == 0 && j >= 8 && j < 12) {
-        long long *f = kcg_fine[threadIdx.x >> 6][j - 8];
-        f[0] = (long long)(f_t0 - f_prev);      // previous end-of-interval barrier wait (t6 of last iteration -> t0)
-        f[1] = (long long)(f_t1 - f_t0);        // softmax
-        f[2] = (long long)(f_t2 - f_t1);        // loads, prefetch, waits
-        f[3] = (long long)(fine_ts[8] - f_t2);  // barrier
-        f[4] = (long long)(fine_ts[7] - fine_ts[8]);  // 32 MFMAs issued
-        f[5] = (long long)(t_b - fine_ts[7]);   // tail
-        f[6] = (long long)(f_t2 & 0xffffff);           // absolute: arrival at the barrier that ends the softmax interval
-        f[7] = (long long)(fine_ts[8] & 0xffffff);     // absolute: first instruction after it
-        f[5] = (long long)(t_b & 0xffffff);            // absolute: arrival at the barrier that ends the matrix interval
-        f[0] = (long long)(f_t0 & 0xffffff);           // absolute: loop top (after the previous barrier)
-      }
-      f_prev = t_b;
-    }
-#endif
+    // group 1 ends the interval in which group 0 reads ahead into the next V tile: its own
+    // share of that tile and of the K tile after it (requested in its last softmax interval
+    // but one) must be in
+    if (group == 1) wait_vm(x_cur + d_cur + x_prev);
     sync();
+    d_prev = d_cur;
+    x_prev2 = x_prev;
+    x_prev = x_cur;
+    x_cur = 0;
+    running = has_next;
   }
   if (group == 0) sync();
 }
@@ -1008,8 +1007,11 @@ static int launch_fmha_bf16_pp(const uint16_t *Q, const uint16_t *K, const uint1
   using T = FmhaPpTile<D>;
   const int64_t q_blocks = (static_cast<int64_t>(S) + T::kBr - 1) / T::kBr;
   const int64_t q_items = causal ? (q_blocks + 1) / 2 : q_blocks;
-  const int64_t blocks = q_items * B * H;
-  if (blocks > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
+  const int64_t items = q_items * B * H;
+  if (items > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
+  // one workgroup per CU (the 144 KiB of LDS allow no second one); each walks its share of
+  // the items as one stream of K/V tiles
+  const int64_t blocks = items < kNumCu ? items : kNumCu;
   if (info) {
     info->grid[0] = static_cast<int>(blocks);
     info->grid[1] = info->grid[2] = 1;
@@ -1025,7 +1027,7 @@ static int launch_fmha_bf16_pp(const uint16_t *Q, const uint16_t *K, const uint1
   auto go = [&](auto kern) {
     if (!allow_lds(kern, T::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
     return launch(kern, dim3(static_cast<unsigned>(blocks)), dim3(T::kThreads), T::kLdsBytes, stream, Q, K, V, O, S,
-                  static_cast<int>(q_blocks), static_cast<int>(q_items), scale_log2e);
+                  static_cast<int>(q_blocks), static_cast<int>(q_items), static_cast<int>(items), scale_log2e);
   };
   const bool obf = o_dtype == KCG_BF16;
   if (causal) return obf ? go(fmha_bf16_pp_kernel<D, true, true>) : go(fmha_bf16_pp_kernel<D, true, false>);
