@@ -1,0 +1,59 @@
+"""Address arithmetic of the direct-load matmul kernel, replayed on the host.
+
+tests/gemm_dl_address_model.cc walks every workgroup, wave and lane of one launch of
+gemm_f32_dl_kernel through the kernel's own integer expressions (it shares the tile
+geometry header with the kernel) and checks that every global byte a direct load, a tail
+re-load or a store of C touches lies inside its tensor, that no 32-bit intermediate
+overflows and that the stores cover C exactly.  No GPU is involved.
+
+The cases include the three launches of the one call that ever ended in a GPU memory
+fault (A = 66000 x 33000, more than 2^31 elements): 65536 rows on the 256 x 128 x 16 tile,
+the remaining 464 rows on 64 x 64 x 32 at A + 65536 * K, and the 488-row call that
+followed.  All three are clean, so the kernel's addressing is not the cause of that
+fault; kcg_gemm_f32 keeps refusing operands of that size class.
+"""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC = os.path.join(ROOT, "tests", "gemm_dl_address_model.cc")
+INC = os.path.join(ROOT, "kernelcodegen_amd", "csrc")
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("gemm_dl") / "gemm_dl_address_model")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-I", INC, SRC, "-o", exe], check=True)
+    return exe
+
+
+# (BM, BN, BK, WAVES_M, WAVES_N, M, N, K, GROUP_M)
+CASES = [
+    # the faulting call, launch by launch
+    (256, 128, 16, 4, 2, 65536, 128, 33000, 8),
+    (64, 64, 32, 2, 2, 464, 128, 33000, 8),
+    (64, 64, 32, 2, 2, 488, 128, 33000, 8),
+    # BASELINE configs on their default tiles
+    (256, 128, 16, 4, 2, 4096, 4096, 4096, 8),
+    (256, 128, 16, 4, 2, 4096, 2048, 1024, 8),
+    (256, 128, 16, 4, 2, 32768, 768, 768, 8),
+    # ragged in every dimension, every built tile
+    (128, 128, 32, 2, 2, 1000, 1000, 1000, 8),
+    (128, 128, 16, 2, 2, 4100, 516, 72, 4),
+    (128, 128, 8, 2, 2, 130, 132, 44, 8),
+    (256, 128, 32, 4, 2, 4100, 4100, 4100, 8),
+    (128, 64, 32, 2, 2, 2050, 2052, 36, 1),
+    (64, 64, 32, 2, 2, 65, 68, 32, 8),
+    # byte offsets beyond 2^32 inside A and inside C
+    (256, 128, 16, 4, 2, 40000, 256, 32768, 8),
+    (128, 64, 32, 2, 2, 40000, 32768, 64, 8),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(map(str, c)))
+def test_every_access_inside_its_tensor(model, case):
+    r = subprocess.run([model] + [str(v) for v in case], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert " 0 violations" in r.stdout

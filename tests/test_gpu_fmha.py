@@ -69,6 +69,43 @@ def test_f32_rising_row_maximum(oracle, dev, causal):
         assert max(rel_err(O, ref)) < TOL_F32, tile
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("which", [0, 1])
+def test_large_logits_in_one_half_of_the_wave(oracle, dev, dtype, which):
+    """The two halves of a wave hold different keys of the same query row (keys with
+    k % 8 < 4 in the lower half, the others in the upper half) and must agree on the row
+    maximum.  Here only one half's keys carry large logits (100 above the rest: 2^144 if
+    the reference were not raised), in every tile; a maximum taken from the other half
+    alone overflows the exponentials."""
+    import torch
+    from kernelcodegen_amd import ops
+    B, H, S, D = 1, 2, 320, 64
+    rng = np.random.default_rng(91)
+    Q = (rng.standard_normal((B, H, S, D)) * 0.05).astype(np.float32)
+    K = (rng.standard_normal((B, H, S, D)) * 0.05).astype(np.float32)
+    V = (rng.standard_normal((B, H, S, D)) + 2.0).astype(np.float32)   # (a mean of many V rows: keep it away from 0)
+    keys = np.arange(S)
+    big = (keys % 8 >= 4) if which else (keys % 8 < 4)
+    Q[..., 0] = 10.0
+    K[..., 0] = np.where(big, 10.0, 0.0)
+    for causal in (False, True):
+        if dtype == "f32":
+            ref = oracle.fmha(Q, K, V, scale=1.0, causal=causal, stable=True)
+            for tile in ((128, 32), (128, 64), (256, 32)):
+                O = ops.fmha(_gpu(Q, dev), _gpu(K, dev), _gpu(V, dev), scale=1.0, causal=causal,
+                             sched=dict(br=tile[0], bc=tile[1])).cpu().numpy()
+                assert np.isfinite(O).all(), tile
+                assert max(rel_err(O, ref)) < TOL_F32, tile
+        else:
+            qb, kb, vb = (inputs.to_bf16_bits(t) for t in (Q, K, V))
+            ref = oracle.fmha(qb, kb, vb, scale=1.0, causal=causal, stable=True)
+            for br in (128, 256):
+                O = ops.fmha(_gpu_bf16(qb, dev), _gpu_bf16(kb, dev), _gpu_bf16(vb, dev), scale=1.0,
+                             causal=causal, out_dtype=torch.float32, sched=dict(br=br, bc=64)).cpu().numpy()
+                assert np.isfinite(O).all(), br
+                assert max(rel_err(O, ref)) < TOL_BF16, br
+
+
 def test_f32_reference_graph_scale_one(oracle, dev):
     """scale = 1, no mask: the reference's own three-operator graph, literal softmax."""
     from kernelcodegen_amd import ops
