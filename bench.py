@@ -7,7 +7,13 @@ resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s, the roofline of the
 kernel (algorithmic FLOPs / HIP-event launch time vs the fp32 MFMA peak), the CPU
 oracle timed on the host cores, and the two attention workloads as extras.
 
+Every timed region is preceded by an untimed clock-settle phase (SETTLE_MS of back-to-back
+launches of the same call) in addition to the --warmup launches, so that the figures do not
+depend on how many warm-up steps the caller asks for.
+
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+    python bench.py --sweep matmul [--max-dim D] [--relu] [--seeded] [--dump DIR]
+    python bench.py --sweep fmha | --sweep ops [--shape B,H,S,D]
 """
 import argparse
 import json
@@ -21,10 +27,22 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 
-# HBM bytes per launch (fetch + write) measured with rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE, each scaled by the same counter's reading for a 256 MiB copy
-# (profiles/gemm_f32_cfg1.md, profiles/fmha_f32_cfg3.md, profiles/fmha_bf16_cfg4.md).
-TRAFFIC_BYTES = {"gemm_cfg1": 744663460, "fmha_cfg3": 138053321, "fmha_cfg4": 795121940}
+# HBM bytes per launch (fetch + write).  NOT measured by this script: counters cannot be
+# read from inside the timed run, so these are the figures of separate rocprofv3 --pmc
+# FETCH_SIZE / --pmc WRITE_SIZE runs of kernelcodegen_amd/profile_kernels.py, each scaled by
+# the same counter's reading for a 256 MiB copy, as recorded in the named profile files.
+TRAFFIC = {
+    "gemm_cfg1": (744663460, "profiles/gemm_f32_cfg1.md"),
+    "fmha_cfg3": (138053321, "profiles/fmha_f32_cfg3.md"),
+    "fmha_cfg4": (795121940, "profiles/fmha_bf16_cfg4.md"),
+}
+
+
+def traffic_fields(key):
+    nbytes, src = TRAFFIC[key]
+    return {"traffic": nbytes,
+            "traffic_source": src + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, copy-calibrated; "
+                                    "a separate run, not measured here)"}
 
 
 def _cpu_model():
@@ -38,10 +56,32 @@ def _cpu_model():
     return "unknown"
 
 
+SETTLE_MS = 40.0   # untimed launches before every timed region, whatever --warmup says
+
+
+def settle(fn, ms=SETTLE_MS):
+    """Runs fn back to back for at least `ms` milliseconds, untimed, and returns the
+    milliseconds spent.  The shader clock drops within a millisecond of idle time (host
+    work, allocations, the CPU leg) and needs tens of milliseconds of load to come back;
+    a handful of warm-up launches of a sub-millisecond kernel is not enough."""
+    import torch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    fn()
+    torch.cuda.synchronize()
+    one = max(time.perf_counter() - t0, 1e-6)
+    for _ in range(min(20000, int(ms * 1e-3 / one) + 1)):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3
+
+
 def time_launches(fn, steps, warmup):
-    """(wall ms per step, HIP-event ms per launch) over `steps` launches of fn."""
+    """(wall ms per step, HIP-event ms per launch) over `steps` launches of fn, after the
+    clock-settle phase and `warmup` further untimed launches."""
     import torch
     stream = torch.cuda.current_stream()
+    settle(fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -79,6 +119,15 @@ def main():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the attention workloads")
+    ap.add_argument("--sweep", choices=["matmul", "fmha", "ops"],
+                    help="instead of the benchmark line, print a measurement sweep: the reference's "
+                         "matmul size sweep in its output.log format, the attention shape grid, or the "
+                         "un-fused operators against their rooflines (kernelcodegen_amd/sweeps.py)")
+    ap.add_argument("--max-dim", type=int, default=16384, help="--sweep matmul: largest square size")
+    ap.add_argument("--relu", action="store_true", help="--sweep matmul: with the fused ReLU epilogue")
+    ap.add_argument("--seeded", action="store_true", help="--sweep matmul: operands from the seeded generator")
+    ap.add_argument("--dump", help="--sweep matmul: directory that receives sampled rows of every C")
+    ap.add_argument("--shape", default="1,32,2048,128", help="--sweep ops: B,H,S,D")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the matmul and attention kernels shard over row "
@@ -95,6 +144,15 @@ def main():
         sys.exit("bench.py needs a GPU")
     lib.load()
     dev = torch.device("cuda:0")
+    if args.sweep:
+        from kernelcodegen_amd import sweeps
+        if args.sweep == "matmul":
+            sweeps.matmul(args.max_dim, args.relu, args.seeded, args.dump)
+        elif args.sweep == "fmha":
+            sweeps.fmha()
+        else:
+            sweeps.ops_chain(tuple(int(x) for x in args.shape.split(",")))
+        return
 
     # ---------------- headline: configs[1], fp32 4096^3 matmul + ReLU ----------------
     cfg = inputs.config_inputs(1)
@@ -118,6 +176,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "clock_settle_ms": SETTLE_MS,
         "ms_per_step": round(wall_ms, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -129,7 +188,7 @@ def main():
         "pct_fp32_peak": round(100.0 * value / PEAK_FP32_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_TFLOPS, 4),
-                     "traffic": TRAFFIC_BYTES["gemm_cfg1"], "kernel": "gemm_f32_dl_kernel",
+                     **traffic_fields("gemm_cfg1"), "kernel": "gemm_f32_dl_kernel",
                      "algorithmic_flops": flops, "algorithmic_bytes": alg_bytes,
                      "launch_ms": round(ev_ms, 5), "launch_ms_median": round(med_ms, 5),
                      "launch_ms_min": round(min_ms, 5)},
@@ -159,10 +218,8 @@ def main():
     # ---------------- extras: the two attention workloads ----------------
     if not args.no_extras:
         extras = {}
-        # the shader clock needs some tens of milliseconds of load to settle after the idle
-        # time of the CPU baseline: the sub-millisecond attention launches get extra warm-up
         steps = max(5, args.steps)
-        warm = max(args.warmup, 50)
+        warm = args.warmup
         c3 = inputs.config_inputs(3)
         Q, Kt, V = (torch.from_numpy(c3[k]).to(dev) for k in "QKV")
         O = torch.empty_like(Q)
@@ -176,7 +233,7 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(fl / (e * 1e-3) / 1e12, 3),
                          "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(fl / (e * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4),
-                         "traffic": TRAFFIC_BYTES["fmha_cfg3"]}}
+                         **traffic_fields("fmha_cfg3")}}
         del Q, Kt, V, O
         c4 = inputs.config_inputs(4)
         Q, Kt, V = (torch.from_numpy(c4[k].view(np.int16)).to(dev).view(torch.bfloat16) for k in "QKV")
@@ -191,7 +248,7 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(fl / (e * 1e-3) / 1e12, 3),
                          "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(fl / (e * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-                         "traffic": TRAFFIC_BYTES["fmha_cfg4"]}}
+                         **traffic_fields("fmha_cfg4")}}
         out["extras"] = extras
 
     print(json.dumps(out))

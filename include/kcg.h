@@ -74,6 +74,13 @@ typedef struct kcg_gemm_sched {
   int32_t wave_n;    /* columns of C per wavefront (THREAD_SIZE_N analogue)    */
   int32_t vec_width; /* VECTORIZE_WIDTH: floats per global/LDS access (4)      */
   int32_t wave_size; /* WARP_SIZE: must be 64 (or 0) on gfx950                 */
+  int32_t lds_stages;/* copies of the K-slice tiles held in LDS, i.e. the leading
+                      * dimension Rewriter::pipeline gives the shared buffers
+                      * (src/Optimizer/Rewriter.cc:809-1180; the reference's
+                      * schedule has 2).  2: slices staged through registers into
+                      * double-buffered LDS; 3: ring of three filled by direct
+                      * global->LDS loads (needs 16-byte aligned rows, K >= block_k);
+                      * 0: the library chooses (3 where the shape allows, else 2). */
 } kcg_gemm_sched;
 
 /* C[M,N] = epilogue(A[M,K] . B[K,N]); fp32, row-major, contiguous.
@@ -96,8 +103,20 @@ typedef struct kcg_launch_info {
   int32_t lds_bytes;
   int32_t waves_per_block;
   char kernel[64];
+  /* A matmul whose tile count leaves the last round of workgroups nearly empty is run as
+   * two launches on the same stream: `main_rows` rows of C on the tile above, the
+   * remaining `tail_rows` on a smaller tile.  launches == 1: the tail_* fields are 0. */
+  int32_t launches;
+  int32_t main_rows;
+  int32_t tail_rows;
+  int32_t tail_grid[3];
+  int32_t tail_block[3];
+  int32_t tail_lds_bytes;
+  char tail_kernel[64];
 } kcg_launch_info;
 
+/* Applies the same shape checks as kcg_gemm_f32 (a shape that call refuses is refused
+ * here with the same status). */
 KCG_API int kcg_gemm_f32_query(int64_t M, int64_t N, int64_t K,
                                const kcg_gemm_sched *sched, kcg_launch_info *out);
 
@@ -156,7 +175,10 @@ KCG_API int kcg_batched_matmul_f32(const float *A, int transA, const float *B,
                                    int64_t N, int64_t K, void *stream);
 
 /* In-place softmax over the last axis of a [rows, n] tensor:
- * x = exp(x) / sum(exp(x)).  src/Frontend/Operators.cc:425-542. */
+ * x = exp(x) / sum(exp(x)), src/Frontend/Operators.cc:425-542 -- evaluated as
+ * exp(x - max) / sum(exp(x - max)), which is the same number by shift invariance wherever
+ * the reference's literal form is finite, and stays finite where that form overflows
+ * (x > 88 gives inf / inf = NaN there).  A deliberate deviation. */
 KCG_API int kcg_softmax_f32(float *x, int64_t rows, int64_t n, void *stream);
 
 #ifdef __cplusplus

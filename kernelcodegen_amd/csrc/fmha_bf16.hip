@@ -970,6 +970,8 @@ static int launch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t
   const int64_t blocks = q_items * B * H;
   if (blocks > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
   if (info) {
+    *info = kcg_launch_info{};
+    info->launches = 1;
     info->grid[0] = static_cast<int>(blocks);
     info->grid[1] = info->grid[2] = 1;
     info->block[0] = T::kThreads;
@@ -1013,6 +1015,8 @@ static int launch_fmha_bf16_pp(const uint16_t *Q, const uint16_t *K, const uint1
   // the items as one stream of K/V tiles
   const int64_t blocks = items < kNumCu ? items : kNumCu;
   if (info) {
+    *info = kcg_launch_info{};
+    info->launches = 1;
     info->grid[0] = static_cast<int>(blocks);
     info->grid[1] = info->grid[2] = 1;
     info->block[0] = T::kThreads;

@@ -348,6 +348,8 @@ static int launch_fmha_f32(const float *Q, const float *K, const float *V, float
   const int64_t blocks = q_items * B * H;
   if (blocks > 0x7fffffffLL) return KCG_ERR_BAD_SHAPE;
   if (info) {
+    *info = kcg_launch_info{};
+    info->launches = 1;
     info->grid[0] = static_cast<int>(blocks);
     info->grid[1] = info->grid[2] = 1;
     info->block[0] = T::kThreads;

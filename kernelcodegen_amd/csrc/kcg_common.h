@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <tuple>
 #include <utility>
 
@@ -106,12 +107,34 @@ inline int launch(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_byte
   return launch_impl(kern, grid, block, lds_bytes, stream, packed, std::index_sequence_for<KArgs...>{});
 }
 
-// Kernels that need more than 48 KiB of dynamic LDS must opt in once per function.
+// Kernels that need more than 48 KiB of dynamic LDS must opt in, once per function and
+// device.  The opt-in is a runtime call of a few microseconds -- as long as the smallest
+// matmuls run -- so it is made on a kernel's first launch only and remembered in a small
+// lock-free table (thread safe; a lost race merely repeats the call).
+inline bool lds_opt_in_once(const void *kern, int lds_bytes) {
+  constexpr int kSlots = 256;
+  static std::atomic<uintptr_t> seen[kSlots];  // zero-initialised: empty
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return false;
+  // kernel addresses are at least 4-byte aligned code addresses well below 2^56
+  const uintptr_t key = reinterpret_cast<uintptr_t>(kern) ^ (static_cast<uintptr_t>(device + 1) << 56);
+  for (int i = 0; i < kSlots; ++i) {
+    const uintptr_t v = seen[i].load(std::memory_order_acquire);
+    if (v == key) return true;
+    if (v == 0) break;
+  }
+  if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) return false;
+  for (int i = 0; i < kSlots; ++i) {
+    uintptr_t expected = 0;
+    if (seen[i].compare_exchange_strong(expected, key, std::memory_order_acq_rel) || expected == key) break;
+  }
+  return true;  // (a full table only means the call is repeated next time)
+}
+
 template <typename... KArgs>
 inline bool allow_lds(void (*kern)(KArgs...), int lds_bytes) {
   if (lds_bytes <= 48 * 1024) return true;
-  return hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) == hipSuccess;
+  return lds_opt_in_once(reinterpret_cast<const void *>(kern), lds_bytes);
 }
 
 // Defined in gemm_f32.hip: BatchedMatmul with A as [batch][M][K] and B as [batch][K][N] or

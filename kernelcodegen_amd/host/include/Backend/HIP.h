@@ -30,6 +30,12 @@ struct KernelBinding {
   int64_t M = 0, N = 0, K = 0;
   int epilogue = KCG_EPILOGUE_NONE;
   kcg_gemm_sched gemmSched{};
+  // Where block_k, lds_stages and vec_width came from: "ir" when the function carries a
+  // staged or pipelined schedule (they are then read off the scheduled loop nest: the
+  // extents of the shared tiles, the leading dimension Rewriter::pipeline gave them, the
+  // width of the vector accesses), "attributes" for a nest that stops at the tiling stage.
+  std::string scheduleSource = "attributes";
+  std::string scheduleNote;   // anything the binding changed, in words (empty: nothing)
   // attention
   int B = 0, H = 0, S = 0, D = 0;
   int dtype = KCG_F32;

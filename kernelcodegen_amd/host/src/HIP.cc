@@ -1,10 +1,13 @@
 #include "Backend/HIP.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <iostream>
+#include <set>
 #include <sstream>
 
 #include "Optimizer/Analyzer.h"
+#include "enum.h"
 
 namespace KernelCodeGen {
 
@@ -17,6 +20,60 @@ int attrInt(FuncOp f, const std::string &key, int fallback) {
   return v.empty() ? fallback : std::stoi(v);
 }
 
+// What the scheduled loop nest of a matmul function says about the kernel: read off the
+// IR, not off the kcg.* attributes.  The reference's backend prints whatever nest the
+// Rewriter calls left behind (split(k) -> BLOCK_SIZE_K, pipeline -> two copies of each
+// shared tile, vectorize -> float4 accesses; src/Optimizer/Optimizer.cc:494-519,
+// src/Optimizer/Rewriter.cc:786-1180); here the same facts select the prebuilt kernel.
+struct NestSchedule {
+  bool staged = false;      // the nest holds shared-memory tiles at all
+  int64_t bk = 0;           // rows of the shared tiles = the k-split factor
+  std::vector<int64_t> tileExtents;  // their columns: BLOCK_SIZE_M and BLOCK_SIZE_N
+  int64_t copies = 0;       // leading dimension added by pipeline (1 without it)
+  int vec = 0;              // width of the vector loads / stores (0: none)
+  std::string problem;      // non-empty: the nest is not one the library can bind
+};
+
+NestSchedule readNestSchedule(FuncOp f) {
+  NestSchedule n;
+  std::vector<MemRefType> shared;
+  std::set<int> widths;
+  walk(f.op, [&](Op *o) {
+    if (o->kind == OpKind::Alloc && !o->results.empty()) {
+      const MemRefType &t = o->result().getMemRefType();
+      if (t.space == static_cast<int>(MemorySpace::shared)) shared.push_back(t);
+    }
+    if ((o->kind == OpKind::Load || o->kind == OpKind::Store) && o->vec > 1) widths.insert(o->vec);
+  });
+  if (shared.empty()) return n;
+  n.staged = true;
+  if (shared.size() != 2) {
+    n.problem = "expected one shared tile of A and one of B, found " + std::to_string(shared.size());
+    return n;
+  }
+  for (const MemRefType &t : shared) {
+    if (t.shape.size() != 2 && t.shape.size() != 3) {
+      n.problem = "shared tile " + t.str() + " is neither [BK][B] nor [copies][BK][B]";
+      return n;
+    }
+    const int64_t copies = t.shape.size() == 3 ? t.shape[0] : 1;
+    const int64_t bk = t.shape[t.shape.size() - 2];
+    if ((n.copies && n.copies != copies) || (n.bk && n.bk != bk)) {
+      n.problem = "the shared tiles of A and B disagree on BLOCK_SIZE_K or on the number of copies";
+      return n;
+    }
+    n.copies = copies;
+    n.bk = bk;
+    n.tileExtents.push_back(t.shape.back());
+  }
+  if (widths.size() > 1) {
+    n.problem = "vector accesses of different widths";
+    return n;
+  }
+  n.vec = widths.empty() ? 0 : *widths.begin();
+  return n;
+}
+
 bool bindMatmul(FuncOp f, KernelBinding &b) {
   auto args = f.getArguments();
   if (args.size() != 3) return false;
@@ -24,6 +81,11 @@ bool bindMatmul(FuncOp f, KernelBinding &b) {
   const auto &tb = args[1].getMemRefType();
   if (ta.elem != DType::f32 || tb.elem != DType::f32 || ta.shape.size() != 2 || tb.shape.size() != 2) {
     std::cerr << "HIPBind: " << f.getSymName() << ": only float32 rank-2 matmul has a gfx950 kernel\n";
+    return false;
+  }
+  if (ta.shape[1] != tb.shape[0]) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": A is " << ta.shape[0] << " x " << ta.shape[1] << " but B is "
+              << tb.shape[0] << " x " << tb.shape[1] << " (K extents differ)\n";
     return false;
   }
   b.kind = KernelBinding::Gemm;
@@ -41,6 +103,37 @@ bool bindMatmul(FuncOp f, KernelBinding &b) {
   b.gemmSched.vec_width = attrInt(f, "kcg.VECTORIZE_WIDTH", 0);
   b.gemmSched.wave_size = attrInt(f, "kcg.WARP_SIZE", 0);
   b.argNames = {"A", "B", "C"};
+  // A staged / pipelined nest decides block_k, the LDS buffer count and the vector width
+  // itself; the attributes must not contradict it.
+  const NestSchedule nest = readNestSchedule(f);
+  if (!nest.problem.empty()) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": " << nest.problem << "\n";
+    return false;
+  }
+  if (nest.staged) {
+    std::vector<int64_t> want = {b.gemmSched.block_m, b.gemmSched.block_n}, got = nest.tileExtents;
+    std::sort(want.begin(), want.end());
+    std::sort(got.begin(), got.end());
+    if (got != want || (b.gemmSched.block_k && b.gemmSched.block_k != nest.bk) ||
+        (nest.vec && b.gemmSched.vec_width && b.gemmSched.vec_width != nest.vec)) {
+      std::cerr << "HIPBind: " << f.getSymName() << ": the scheduled nest (shared tiles " << nest.bk << " x {"
+                << nest.tileExtents[0] << ", " << nest.tileExtents[1] << "}, vector width " << nest.vec
+                << ") contradicts the kcg.* attributes (" << b.gemmSched.block_m << " x " << b.gemmSched.block_n
+                << " x " << b.gemmSched.block_k << ", width " << b.gemmSched.vec_width << ")\n";
+      return false;
+    }
+    b.scheduleSource = "ir";
+    b.gemmSched.block_k = static_cast<int>(nest.bk);
+    if (nest.vec) b.gemmSched.vec_width = nest.vec;
+    if (nest.copies == 1) {
+      // a single-buffered schedule: the library's least-buffered kernel holds two copies
+      b.gemmSched.lds_stages = 2;
+      b.scheduleNote = "the nest keeps one copy of each shared tile; run on the double-buffered kernel "
+                       "(the library builds no single-buffered one)";
+    } else {
+      b.gemmSched.lds_stages = static_cast<int>(nest.copies);
+    }
+  }
   const int st = kcg_gemm_f32_query(b.M, b.N, b.K, &b.gemmSched, &b.launch);
   if (st != KCG_OK) {
     std::cerr << "HIPBind: " << f.getSymName() << ": " << kcg_status_str(st) << "\n";
@@ -125,11 +218,24 @@ std::string HIPGen(ModuleOp &module) {
        << "), block dims:(" << b.launch.block[0] << ", " << b.launch.block[1] << ", " << b.launch.block[2]
        << "), lds bytes:" << b.launch.lds_bytes << "\n";
     if (b.kind == KernelBinding::Gemm) {
+      os << "// block_k " << b.gemmSched.block_k << ", lds stages " << b.gemmSched.lds_stages << " (0 = library's choice)"
+         << ", vector width " << b.gemmSched.vec_width << ": from the " << (b.scheduleSource == "ir" ? "scheduled loop nest" : "kcg.* attributes")
+         << "\n";
+      if (!b.scheduleNote.empty()) os << "// note: " << b.scheduleNote << "\n";
+    }
+    if (b.launch.launches == 2)
+      os << "// first launch: rows 0.." << b.launch.main_rows - 1 << "; second launch (" << b.launch.tail_kernel
+         << "): the last " << b.launch.tail_rows << " rows, grid dims:(" << b.launch.tail_grid[0] << ", "
+         << b.launch.tail_grid[1] << ", " << b.launch.tail_grid[2] << "), block dims:(" << b.launch.tail_block[0]
+         << ", " << b.launch.tail_block[1] << ", " << b.launch.tail_block[2] << "), lds bytes:"
+         << b.launch.tail_lds_bytes << "\n";
+    if (b.kind == KernelBinding::Gemm) {
       os << "inline int kernel" << b.index
          << "(const float* arg0 /*A*/, const float* arg1 /*B*/, float* arg2 /*C*/, void* stream = nullptr) {\n"
          << "  static const kcg_gemm_sched sched = {" << b.gemmSched.block_m << ", " << b.gemmSched.block_n << ", "
          << b.gemmSched.block_k << ", " << b.gemmSched.group_m << ", " << b.gemmSched.wave_m << ", "
-         << b.gemmSched.wave_n << ", " << b.gemmSched.vec_width << ", " << b.gemmSched.wave_size << "};\n"
+         << b.gemmSched.wave_n << ", " << b.gemmSched.vec_width << ", " << b.gemmSched.wave_size << ", "
+         << b.gemmSched.lds_stages << "};\n"
          << "  return kcg_gemm_f32(arg0, arg1, arg2, " << b.M << ", " << b.N << ", " << b.K << ", "
          << (b.epilogue == KCG_EPILOGUE_RELU ? "KCG_EPILOGUE_RELU" : "KCG_EPILOGUE_NONE") << ", &sched, stream);\n"
          << "}\n\n";

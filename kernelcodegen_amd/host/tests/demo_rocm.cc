@@ -2,6 +2,11 @@
 // flows (test/test.cc:8-107 there) carried through to a launch on the device.
 //
 //   demo_rocm matmul M N K relu(0|1) out.bin
+//   demo_rocm sched  M N K relu(0|1) detail(0|1|2) out.bin   the reference's 128 x 128 x 8 tile
+//                    with the staged (1) or pipelined (2) schedule built on the IR: the
+//                    binding reads block_k, the LDS buffer count and the vector width off
+//                    the scheduled nest ("schedule <source> block_k <n> lds_stages <n>
+//                    vec_width <n>" is printed)
 //   demo_rocm fmha   B H S D causal(0|1) scale out.bin
 //   demo_rocm tune matmul M N K relu(0|1) out.bin
 //   demo_rocm tune fmha   B H S D causal(0|1) scale out.bin
@@ -113,7 +118,16 @@ int main(int argc, char **argv) {
       std::printf("best %s %.5f\n", sched, generator.bestLatency());
     }
   };
-  const std::string mode = argv[1];
+  std::string mode = argv[1];
+  if (mode == "sched" && argc == 8) {
+    const int detail = std::atoi(argv[6]);
+    generator.matmulConfigs = {{{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 8}, {"GROUP_SIZE_M", 8},
+                                {"THREAD_SIZE_M", 8}, {"THREAD_SIZE_N", 8}, {"WAVE_SIZE_M", 64}, {"WAVE_SIZE_N", 64},
+                                {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64}, {"SCHEDULE_DETAIL", detail}}};
+    argv[6] = argv[7];
+    --argc;
+    mode = "matmul";
+  }
   if (mode == "matmul" && argc == 7) {
     const int64_t m = std::atoll(argv[2]), n = std::atoll(argv[3]), k = std::atoll(argv[4]);
     const bool relu = std::atoi(argv[5]) != 0;
@@ -126,6 +140,9 @@ int main(int argc, char **argv) {
     auto bindings = generator.bind(module);
     if (bindings.size() != 1) return 5;
     report(bindings);
+    std::printf("schedule %s block_k %d lds_stages %d vec_width %d kernel %s\n", bindings[0].scheduleSource.c_str(),
+                bindings[0].gemmSched.block_k, bindings[0].gemmSched.lds_stages, bindings[0].gemmSched.vec_width,
+                bindings[0].launch.kernel);
     std::printf("%s", generator.codegen(module).c_str());
     std::vector<float> a(m * k), b(k * n);
     fill_uniform(a, kSeed, 0);

@@ -711,6 +711,86 @@ static void test_facade_matmul_demo() {
   CHECK(none.empty());
 }
 
+// The scheduled nest drives the binding: block_k is the extent the k split left on the
+// shared tiles, the LDS buffer count is the leading dimension pipeline() gave them, the
+// vector width is that of the vectorised accesses -- and a nest that contradicts the
+// kcg.* attributes is refused.
+static void test_schedule_drives_binding() {
+  auto bindWith = [](int detail, ir::ModuleOp *keep = nullptr) {
+    KernelCodeGenerator generator("ROCm");
+    generator.setLogMode(Log::Release);
+    generator.matmulConfigs = {{{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 8}, {"GROUP_SIZE_M", 8},
+                                {"THREAD_SIZE_M", 8}, {"THREAD_SIZE_N", 8}, {"WAVE_SIZE_M", 64}, {"WAVE_SIZE_N", 64},
+                                {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64}, {"SCHEDULE_DETAIL", detail}}};
+    auto &graph = generator.createGraph("sched_demo");
+    auto A = graph.create<PlaceHolder>(std::vector<int64_t>{512, 256}, std::string{"float32"});
+    auto B = graph.create<PlaceHolder>(std::vector<int64_t>{256, 384}, std::string{"float32"});
+    graph.create<Matmul>(A, B, MemorySpace::global);
+    auto module = generator.optimize(graph);
+    auto bindings = generator.bind(module);
+    std::string source = generator.codegen(module);
+    if (keep) *keep = module;
+    return std::make_pair(bindings, source);
+  };
+  {  // tiling stage only: the attributes speak, the library picks the buffer count
+    auto [b, src] = bindWith(0);
+    CHECK(b.size() == 1);
+    if (b.size() == 1) {
+      CHECK(b[0].scheduleSource == "attributes" && b[0].gemmSched.lds_stages == 0 && b[0].gemmSched.block_k == 8);
+      CHECK(std::string(b[0].launch.kernel) == "gemm_f32_128x128x8_w2x2_dl");
+      CHECK(contains(src, "from the kcg.* attributes"));
+    }
+  }
+  {  // staged: one copy of each shared tile -> the double-buffered kernel, with a note
+    auto [b, src] = bindWith(1);
+    CHECK(b.size() == 1);
+    if (b.size() == 1) {
+      CHECK(b[0].scheduleSource == "ir" && b[0].gemmSched.block_k == 8 && b[0].gemmSched.vec_width == 4);
+      CHECK(b[0].gemmSched.lds_stages == 2 && !b[0].scheduleNote.empty());
+      CHECK(std::string(b[0].launch.kernel) == "gemm_f32_128x128x8_w2x2");
+      CHECK(b[0].launch.lds_bytes == 2 * (128 * (8 + 4) + 8 * (128 + 8)) * 4);
+      CHECK(contains(src, "lds stages 2") && contains(src, "from the scheduled loop nest") && contains(src, "// note: "));
+      CHECK(contains(src, "sched = {128, 128, 8, 8, 64, 64, 4, 64, 2};"));
+    }
+  }
+  ir::ModuleOp pipelined;
+  {  // pipelined: memref<2x8x128xf32, 2> tiles -> two LDS stages, no note
+    auto [b, src] = bindWith(2, &pipelined);
+    CHECK(b.size() == 1);
+    if (b.size() == 1) {
+      CHECK(b[0].scheduleSource == "ir" && b[0].gemmSched.lds_stages == 2 && b[0].scheduleNote.empty());
+      CHECK(std::string(b[0].launch.kernel) == "gemm_f32_128x128x8_w2x2");
+      CHECK(contains(pipelined.str(), "memref<2x8x128xf32, 2>"));
+    }
+  }
+  {  // the attributes must not contradict the nest
+    FuncOp f = Analyzer::collectFunctions(pipelined, "Matmul_m")[0];
+    f.setAttr("kcg.BLOCK_SIZE_K", "16");
+    std::vector<KernelBinding> b;
+    quiet([&] { b = HIPBind(pipelined); });
+    CHECK(b.empty());
+    f.setAttr("kcg.BLOCK_SIZE_K", "8");
+    f.setAttr("kcg.VECTORIZE_WIDTH", "2");
+    quiet([&] { b = HIPBind(pipelined); });
+    CHECK(b.empty());
+    f.setAttr("kcg.VECTORIZE_WIDTH", "4");
+    quiet([&] { b = HIPBind(pipelined); });
+    CHECK(b.size() == 1);
+  }
+  {  // the library's own refusals: a buffer count it does not build, the ring on an unaligned shape
+    kcg_launch_info info;
+    kcg_gemm_sched s = {128, 128, 8, 8, 64, 64, 4, 64, 4};
+    CHECK(kcg_gemm_f32_query(512, 384, 256, &s, &info) == KCG_ERR_BAD_SCHEDULE);
+    s.lds_stages = 1;
+    CHECK(kcg_gemm_f32_query(512, 384, 256, &s, &info) == KCG_ERR_BAD_SCHEDULE);
+    s.lds_stages = 3;
+    CHECK(kcg_gemm_f32_query(512, 384, 256, &s, &info) == KCG_OK && contains(info.kernel, "_dl"));
+    CHECK(kcg_gemm_f32_query(512, 384, 250, &s, &info) == KCG_ERR_BAD_SCHEDULE);  // rows not 16-byte aligned
+    s.lds_stages = 2;
+    CHECK(kcg_gemm_f32_query(512, 384, 250, &s, &info) == KCG_OK && !contains(info.kernel, "_dl"));
+  }
+}
+
 static void test_facade_config_search_and_reference_tile() {
   KernelCodeGenerator generator;
   generator.setLogMode(Log::Release);
@@ -897,6 +977,7 @@ int main() {
       {"fused_attention_nest", test_fused_attention_nest},
       {"fmha_pattern_rejections", test_fmha_pattern_rejections},
       {"facade_matmul_demo", test_facade_matmul_demo},
+      {"schedule_drives_binding", test_schedule_drives_binding},
       {"facade_config_search_and_reference_tile", test_facade_config_search_and_reference_tile},
       {"facade_flash_attention_demo", test_facade_flash_attention_demo},
       {"error_paths", test_error_paths},

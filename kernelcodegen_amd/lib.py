@@ -25,7 +25,8 @@ class KcgError(RuntimeError):
 class GemmSched(ctypes.Structure):
     """kcg_gemm_sched: the reference's matmul tile table (include/KernelCodeGen.h:34-37)."""
     _fields_ = [("block_m", _i32), ("block_n", _i32), ("block_k", _i32), ("group_m", _i32),
-                ("wave_m", _i32), ("wave_n", _i32), ("vec_width", _i32), ("wave_size", _i32)]
+                ("wave_m", _i32), ("wave_n", _i32), ("vec_width", _i32), ("wave_size", _i32),
+                ("lds_stages", _i32)]
 
 
 class FmhaSched(ctypes.Structure):
@@ -35,7 +36,10 @@ class FmhaSched(ctypes.Structure):
 
 class LaunchInfo(ctypes.Structure):
     _fields_ = [("grid", _i32 * 3), ("block", _i32 * 3), ("lds_bytes", _i32),
-                ("waves_per_block", _i32), ("kernel", ctypes.c_char * 64)]
+                ("waves_per_block", _i32), ("kernel", ctypes.c_char * 64),
+                ("launches", _i32), ("main_rows", _i32), ("tail_rows", _i32),
+                ("tail_grid", _i32 * 3), ("tail_block", _i32 * 3), ("tail_lds_bytes", _i32),
+                ("tail_kernel", ctypes.c_char * 64)]
 
 
 # name -> (restype, argtypes); every symbol include/kcg.h declares.

@@ -27,6 +27,21 @@ def _dev_f32(t, name):
         raise ValueError("%s must be a contiguous fp32 device tensor" % name)
 
 
+def _check(t, name, dtype, shape, device):
+    """The kernels take raw pointers: a tensor of another dtype, shape, device or layout
+    would make them read or write out of bounds, so it is refused here."""
+    if not isinstance(t, torch.Tensor):
+        raise ValueError("%s must be a tensor" % name)
+    if not t.is_cuda or t.device != device:
+        raise ValueError("%s must be on device %s" % (name, device))
+    if t.dtype != dtype:
+        raise ValueError("%s must have dtype %s, not %s" % (name, dtype, t.dtype))
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError("%s must have shape %s, not %s" % (name, tuple(shape), tuple(t.shape)))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+
+
 def _sched(sched, cls):
     if sched is None:
         return None
@@ -43,9 +58,11 @@ def matmul(A, B, relu=False, out=None, sched=None):
     K2, N = B.shape
     if K != K2:
         raise ValueError("Can't apply Matmul Operation due to imcompatible K-dim.")
+    if B.device != A.device:
+        raise ValueError("A and B must be on the same device")
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=A.device)
-    _dev_f32(out, "out")
+    _check(out, "out", torch.float32, (M, N), A.device)
     st = lib.load().kcg_gemm_f32(_ptr(A), _ptr(B), _ptr(out), M, N, K,
                                  EPILOGUE_RELU if relu else EPILOGUE_NONE,
                                  _sched(sched, lib.GemmSched), lib.current_stream())
@@ -57,8 +74,8 @@ def relu(x, inplace=False, out=None):
     _dev_f32(x, "x")
     if out is not None:
         _dev_f32(out, "out")
-        if out.numel() != x.numel():
-            raise ValueError("relu: out must have as many elements as x")
+        if out.numel() != x.numel() or out.device != x.device:
+            raise ValueError("relu: out must have as many elements as x, on the same device")
     y = x if inplace else (out if out is not None else torch.empty_like(x))
     lib.check(lib.load().kcg_relu_f32(_ptr(x), _ptr(y), x.numel(), lib.current_stream()))
     return y
@@ -78,8 +95,11 @@ def batched_matmul(A, B, trans_a=False, trans_b=False, out=None):
     batch = 1
     for d in batch_shape:
         batch *= d
+    if B.device != A.device:
+        raise ValueError("A and B must be on the same device")
     if out is None:
         out = torch.empty(batch_shape + (M, N), dtype=torch.float32, device=A.device)
+    _check(out, "out", torch.float32, batch_shape + (M, N), A.device)
     st = lib.load().kcg_batched_matmul_f32(_ptr(A), int(trans_a), _ptr(B), int(trans_b), _ptr(out),
                                            batch, M, N, K, lib.current_stream())
     lib.check(st)
@@ -100,25 +120,39 @@ def fmha(Q, K, V, scale=1.0, causal=False, out=None, out_dtype=None, sched=None)
     fp32 tensors run the fp32 kernel; bf16 tensors the bf16 kernel (fp32
     accumulation and softmax), writing `out_dtype` (bf16 by default).
     """
-    if not (Q.is_cuda and Q.is_contiguous() and K.is_contiguous() and V.is_contiguous()):
-        raise ValueError("Q, K, V must be contiguous device tensors")
-    if Q.shape != K.shape or Q.shape != V.shape or Q.dim() != 4:
+    if not isinstance(Q, torch.Tensor) or Q.dim() != 4:
         raise ValueError("Q, K, V must share one [B,H,S,D] shape")
+    if Q.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("fmha supports float32 and bfloat16")
+    if not Q.is_cuda:
+        raise ValueError("Q, K, V must be contiguous device tensors")
+    for t, name in ((Q, "Q"), (K, "K"), (V, "V")):
+        _check(t, name, Q.dtype, Q.shape, Q.device)
     B_, H, S, D = Q.shape
+    if Q.dtype == torch.float32:
+        if out_dtype not in (None, torch.float32):
+            raise ValueError("fp32 attention writes fp32: out_dtype must be float32")
+        want = torch.float32
+    else:
+        if out_dtype not in (None, torch.bfloat16, torch.float32):
+            raise ValueError("bf16 attention writes bfloat16 or float32, not %s" % out_dtype)
+        want = out_dtype or (out.dtype if out is not None else torch.bfloat16)
+        if want not in (torch.bfloat16, torch.float32):
+            raise ValueError("out must be bfloat16 or float32, not %s" % want)
+    if out is not None:
+        _check(out, "out", want, Q.shape, Q.device)
     L = lib.load()
     if Q.dtype == torch.float32:
         if out is None:
             out = torch.empty_like(Q)
         st = L.kcg_fmha_f32(_ptr(Q), _ptr(K), _ptr(V), _ptr(out), B_, H, S, D, float(scale),
                             int(causal), _sched(sched, lib.FmhaSched), lib.current_stream())
-    elif Q.dtype == torch.bfloat16:
+    else:
         if out is None:
-            out = torch.empty(Q.shape, dtype=out_dtype or torch.bfloat16, device=Q.device)
+            out = torch.empty(Q.shape, dtype=want, device=Q.device)
         o_dtype = BF16 if out.dtype == torch.bfloat16 else F32
         st = L.kcg_fmha_bf16(_ptr(Q), _ptr(K), _ptr(V), _ptr(out), o_dtype, B_, H, S, D,
                              float(scale), int(causal), _sched(sched, lib.FmhaSched),
                              lib.current_stream())
-    else:
-        raise ValueError("fmha supports float32 and bfloat16")
     lib.check(st)
     return out

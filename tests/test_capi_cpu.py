@@ -88,9 +88,15 @@ def test_launch_geometry_queries():
     s = lib.GemmSched(block_m=256, block_n=128, block_k=16, wave_m=64, wave_n=64)
     assert L.kcg_gemm_f32_query(7168, 7168, 7168, ctypes.byref(s), ctypes.byref(info)) == 0
     assert info.grid[0] == 28 * 56 and b"+" not in info.kernel
-    # bf16 causal, S = 4096: 256-row query blocks run in pairs (n-1-i, i) -> 8 work items per head
+    # bf16 causal, S = 4096: 256-row query blocks run in pairs (n-1-i, i) -> 8 work items per
+    # head, 1024 in all, walked by one persistent 8-wave workgroup per CU
     assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 1, None, ctypes.byref(info)) == 0
-    assert info.grid[0] == 4 * 32 * 8 and info.block[0] == 512 and info.waves_per_block == 8
+    assert info.grid[0] == 256 and info.block[0] == 512 and info.waves_per_block == 8
+    assert info.kernel == b"fmha_bf16_d128_br256_bc64_pingpong_causal_paired"
+    assert info.lds_bytes == (4 + 5) * 64 * 128 * 2
+    # fewer items than CUs: one workgroup each
+    assert L.kcg_fmha_query(1, 1, 8, 4096, 128, 1, ctypes.byref(lib.FmhaSched(br=256, bc=64)), ctypes.byref(info)) == 0
+    assert info.grid[0] == 8 * 8
     s128 = lib.FmhaSched(br=128, bc=64)
     assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 1, ctypes.byref(s128), ctypes.byref(info)) == 0
     assert info.grid[0] == 4 * 32 * 16 and info.block[0] == 256
@@ -167,3 +173,76 @@ def test_default_matmul_plans_cover_the_problem():
             assert (bm, bn) == (256, 128) and main_rows + int(m.group(4)) == M, (M, N, name)
             assert int(m.group(4)) >= 1
     assert cut > 10      # the sweep's odd multiples of 1024 at least
+
+
+def _meta(shape, dtype, cuda=True, contiguous=True):
+    """A tensor stand-in that carries shape / dtype / device / contiguity only (torch's
+    'meta' tensors report is_cuda False, so the wrappers' checks are driven through a thin
+    subclass instead)."""
+    import torch
+
+    class T(torch.Tensor):
+        @property
+        def is_cuda(self):
+            return cuda
+
+        @property
+        def device(self):
+            return torch.device("cuda:0") if cuda else torch.device("cpu")
+
+        def is_contiguous(self, *a, **k):
+            return contiguous
+
+        def data_ptr(self):
+            raise AssertionError("validation must fail before a pointer is taken")
+
+    return torch.empty(shape, dtype=dtype).as_subclass(T)
+
+
+def test_python_wrappers_refuse_mismatched_tensors():
+    """Every tensor handed to a kernel is checked for device, dtype, contiguity and exact
+    shape first (the kernels only see raw pointers).  None of these calls reaches the GPU."""
+    import torch
+    from kernelcodegen_amd import ops
+    f32, bf16, f16 = torch.float32, torch.bfloat16, torch.float16
+    A, B = _meta((64, 32), f32), _meta((32, 48), f32)
+    with pytest.raises(ValueError):
+        ops.matmul(A, B, out=_meta((64, 40), f32))          # wrong shape
+    with pytest.raises(ValueError):
+        ops.matmul(A, B, out=_meta((64, 48), f16))          # wrong dtype
+    with pytest.raises(ValueError):
+        ops.matmul(A, B, out=_meta((64, 48), f32, cuda=False))
+    with pytest.raises(ValueError):
+        ops.matmul(A, _meta((32, 48), f32, cuda=False))
+    with pytest.raises(ValueError):
+        ops.matmul(A, _meta((31, 48), f32))                 # K mismatch
+    bA, bB = _meta((2, 3, 16, 8), f32), _meta((2, 3, 8, 24), f32)
+    with pytest.raises(ValueError):
+        ops.batched_matmul(bA, bB, out=_meta((2, 3, 16, 20), f32))
+    with pytest.raises(ValueError):
+        ops.batched_matmul(bA, bB, out=_meta((2, 3, 16, 24), bf16))
+    with pytest.raises(ValueError):
+        ops.batched_matmul(bA, bB, out=_meta((2, 3, 16, 24), f32, contiguous=False))
+    shape = (1, 2, 64, 64)
+    Q = _meta(shape, f32)
+    with pytest.raises(ValueError):
+        ops.fmha(Q, _meta(shape, bf16), _meta(shape, f32))  # narrower K: would be read past its end
+    with pytest.raises(ValueError):
+        ops.fmha(Q, _meta(shape, f32, cuda=False), _meta(shape, f32))
+    with pytest.raises(ValueError):
+        ops.fmha(Q, _meta(shape, f32), _meta((1, 2, 64, 32), f32))
+    with pytest.raises(ValueError):
+        ops.fmha(Q, _meta(shape, f32), _meta(shape, f32), out=_meta(shape, bf16))
+    with pytest.raises(ValueError):
+        ops.fmha(Q, _meta(shape, f32), _meta(shape, f32), out_dtype=bf16)
+    Qb, Kb, Vb = (_meta(shape, bf16) for _ in range(3))
+    with pytest.raises(ValueError):
+        ops.fmha(Qb, Kb, Vb, out=_meta(shape, f16))         # 2-byte buffer, would be written as fp32
+    with pytest.raises(ValueError):
+        ops.fmha(Qb, Kb, Vb, out_dtype=f16)
+    with pytest.raises(ValueError):
+        ops.fmha(Qb, Kb, Vb, out=_meta(shape, f32), out_dtype=bf16)   # out disagrees with out_dtype
+    with pytest.raises(ValueError):
+        ops.fmha(Qb, Kb, Vb, out=_meta((1, 2, 64, 32), bf16))
+    with pytest.raises(ValueError):
+        ops.fmha(_meta(shape, f16), _meta(shape, f16), _meta(shape, f16))

@@ -38,6 +38,32 @@ def test_matmul_demo(oracle, dev, tmp_path, shape, relu):
     assert max(rel_err(got.reshape(M, N), ref)) < 1e-4
 
 
+@pytest.mark.parametrize("detail,stages,source", [(0, 0, "attributes"), (1, 2, "ir"), (2, 2, "ir")])
+@pytest.mark.parametrize("shape", [(512, 384, 256), (300, 260, 72)])
+def test_schedule_selects_the_kernel(oracle, dev, tmp_path, shape, detail, stages, source):
+    """The reference's 128 x 128 x 8 tile with the staged (SCHEDULE_DETAIL 1) and pipelined
+    (2) schedules built on the IR: the binding reads block_k, the LDS buffer count and the
+    vector width off the scheduled nest (the shared tiles memref<[2x]8x128xf32, 2>, the
+    float4 accesses), which selects the double-buffered register-staged kernel instead of
+    the library's default three-stage direct-load ring; the launched result is the oracle's."""
+    M, N, K = shape
+    got, text = _run(["sched", M, N, K, 1, detail], tmp_path)
+    m = [l for l in text.splitlines() if l.startswith("schedule ")]
+    assert len(m) == 1
+    f = m[0].split()
+    assert f[1] == source and int(f[3]) == 8 and int(f[5]) == stages and int(f[7]) == 4
+    kernel = f[9]
+    assert kernel.startswith("gemm_f32_128x128x8_w2x2")
+    assert ("_dl" in kernel) == (stages != 2)
+    assert "static const kcg_gemm_sched sched = {128, 128, 8, 8, 64, 64, 4, 64, %d};" % stages in text
+    if detail == 1:
+        assert "// note: the nest keeps one copy of each shared tile" in text
+    A = inputs.uniform((M, K), SEED, 0)
+    B = inputs.uniform((K, N), SEED, 1)
+    ref = oracle.relu(oracle.matmul(A, B))
+    assert max(rel_err(got.reshape(M, N), ref)) < 1e-4
+
+
 @pytest.mark.parametrize("causal", [0, 1])
 def test_flash_attention_demo(oracle, dev, tmp_path, causal):
     B, H, S, D = 2, 4, 384, 64
