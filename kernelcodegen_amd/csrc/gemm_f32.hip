@@ -30,6 +30,7 @@
 #include <type_traits>
 
 #include "gemm_dl_tile.h"
+#include "gemm_f32_stream.h"
 #include "kcg_common.h"
 
 namespace kcg {
@@ -940,8 +941,50 @@ static int launch_bmm_dl(const float *A, const float *B, float *C, int64_t batch
               : go(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, true, MIN_WAVES, false>, lds_bytes);
 }
 
+// The streaming kernel (gemm_f32_stream.h): one resident workgroup per CU walks its share of
+// the (matrix, tile) list.  Taken when every workgroup has at least two tiles to chain.
+static int launch_bmm_stream(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N,
+                             int64_t K, bool trans_b, hipStream_t stream) {
+  using G = GemmStreamGeometry;
+  const int64_t tiles_m = M / G::kBM, tiles_n = N / G::kBN;
+  const int64_t items = tiles_m * tiles_n * batch;
+  const int ctas = static_cast<int>(items < kNumCu ? items : kNumCu);
+  const bool stream_c = M * N * batch > (int64_t{48} << 20);   // C beyond the last-level cache: non-temporal stores
+  auto go = [&](auto kern, int lds_bytes) {
+    if (!allow_lds(kern, lds_bytes)) return static_cast<int>(KCG_ERR_LAUNCH);
+    return launch(kern, dim3(ctas), dim3(512), lds_bytes, stream, A, B, C, static_cast<int>(M), static_cast<int>(N),
+                  static_cast<int>(K), static_cast<int>(tiles_m), static_cast<int>(tiles_n), 8, static_cast<int>(batch),
+                  M * K, K * N, M * N);
+  };
+  auto pick = [&](auto trans_c, auto kt_c) {
+    constexpr bool TB = decltype(trans_c)::value;
+    constexpr int KT = decltype(kt_c)::value;
+    constexpr int lds_bytes =
+        G::kStages * GemmDlTile<G::kBM, G::kBN, G::kBK, G::kWavesM, G::kWavesN, TB>::kStageFloats * 4;
+    return stream_c ? go(gemm_f32_stream_kernel<TB, KT, true>, lds_bytes)
+                    : go(gemm_f32_stream_kernel<TB, KT, false>, lds_bytes);
+  };
+  using K4 = std::integral_constant<int, 4>;
+  using K8 = std::integral_constant<int, 8>;
+  if (trans_b) return K >= 128 ? pick(std::true_type{}, K8{}) : pick(std::true_type{}, K4{});
+  return K >= 128 ? pick(std::false_type{}, K8{}) : pick(std::false_type{}, K4{});
+}
+
+static bool stream_shape(int64_t batch, int64_t M, int64_t N, int64_t K, const float *A, const float *B,
+                         const float *C) {
+  using G = GemmStreamGeometry;
+  if (M % G::kBM || N % G::kBN || K % (4 * G::kBK) || K < 4 * G::kBK) return false;
+  if (N > (1 << 21) || K >= (1 << 22) || M > 0x7fffffffLL) return false;
+  const int64_t items = (M / G::kBM) * (N / G::kBN) * batch;
+  if (items < 2 * kNumCu || items > 0x7fffffffLL) return false;
+  // a long K hides the per-tile prologue and epilogue by itself
+  if (K > 1024) return false;
+  return aligned16(A) && aligned16(B) && aligned16(C);
+}
+
 int dispatch_bmm_dl(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N, int64_t K,
                     bool trans_b, hipStream_t stream) {
+  if (stream_shape(batch, M, N, K, A, B, C)) return launch_bmm_stream(A, B, C, batch, M, N, K, trans_b, stream);
   const kcg_gemm_sched d = default_tile(M, N, batch);
   if (d.block_m == 256) return launch_bmm_dl<256, 128, 16, 4, 2, 2>(A, B, C, batch, M, N, K, trans_b, stream);
   // 128 x 128: the shallow slice has the shorter prologue, which is what counts for the short K

@@ -73,6 +73,51 @@ def test_batched_matmul_direct_load(oracle, dev, tb, dims):
     assert max(rel_err(C, ref)) < 1e-4
 
 
+# Shapes of the streaming kernel (whole 256 x 128 tiles, K a multiple of 64 up to 1024, at least
+# two tiles per compute unit): resident workgroups chain their tiles into one stream of K
+# slices and write each tile's C during the next tile's first slices.  K = 64 and K = 128 are
+# the two store schedules (4 and 8 slices carry stores), 192 and 320 add whole rounds of the
+# slice ring behind them, 1024 is the longest K it takes; tile counts that 8 XCDs x 32
+# workgroups do not divide leave workgroups with lists of different lengths.
+@pytest.mark.parametrize("tb", [True, False])
+@pytest.mark.parametrize("dims", [
+    ((16,), 1024, 1024, 128),
+    ((9,), 1280, 1664, 64),
+    ((3, 3), 1280, 1664, 192),
+    ((20,), 768, 1152, 320),
+    ((5,), 2560, 1408, 1024),
+])
+def test_batched_matmul_streaming_kernel(oracle, dev, tb, dims):
+    import torch
+    from kernelcodegen_amd import ops
+    batch, M, N, K = dims
+    A = inputs.normal(batch + (M, K), 313, 0)
+    B = inputs.normal(batch + ((N, K) if tb else (K, N)), 313, 1)
+    ref = oracle.batched_matmul(A, False, B, tb)
+    count = int(np.prod(batch)) * M * N
+    buf = torch.full((count + 1024,), -7.0, device=dev)
+    C = buf[:count].view(batch + (M, N))
+    ops.batched_matmul(_gpu(A, dev), _gpu(B, dev), trans_b=tb, out=C)
+    assert bool((buf[count:] == -7.0).all())
+    assert max(rel_err(C.cpu().numpy(), ref)) < 1e-4
+
+
+def test_streaming_kernel_result_is_the_tiled_kernels(dev):
+    """The attention-score product at the configs[3] shape on the streaming kernel, against the
+    same product computed one matrix at a time (32 tiles per call: the one-tile-per-workgroup
+    kernel).  Same tile, same slice order, same MFMA operand mapping: the results are equal
+    bit for bit."""
+    import torch
+    from kernelcodegen_amd import ops
+    H, S, D = 32, 2048, 128
+    Q = torch.randn(H, S, D, device=dev)
+    K = torch.randn(H, S, D, device=dev)
+    P = ops.batched_matmul(Q, K, trans_b=True)
+    for h in (0, 13, 31):
+        one = ops.batched_matmul(Q[h:h + 1], K[h:h + 1], trans_b=True)
+        assert torch.equal(P[h], one[0])
+
+
 @pytest.mark.parametrize("K", [32, 3])
 def test_batched_matmul_more_matrices_than_one_launch_takes(dev, K):
     """70000 small matrices: more than the 65535 a launch holds in its grid (K = 32 on the
