@@ -34,7 +34,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 TRAFFIC = {
     "gemm_cfg1": (744663460, "profiles/gemm_f32_cfg1.md"),
     "fmha_cfg3": (138053321, "profiles/fmha_f32_cfg3.md"),
-    "fmha_cfg4": (795121940, "profiles/fmha_bf16_cfg4.md"),
+    "fmha_cfg4": (787606226, "profiles/fmha_bf16_cfg4.md"),
 }
 
 
@@ -60,19 +60,17 @@ SETTLE_MS = 40.0   # untimed launches before every timed region, whatever --warm
 
 
 def settle(fn, ms=SETTLE_MS):
-    """Runs fn back to back for at least `ms` milliseconds, untimed, and returns the
-    milliseconds spent.  The shader clock drops within a millisecond of idle time (host
-    work, allocations, the CPU leg) and needs tens of milliseconds of load to come back;
-    a handful of warm-up launches of a sub-millisecond kernel is not enough."""
+    """Runs fn back to back, untimed, until at least `ms` milliseconds have passed, and
+    returns the milliseconds spent.  The shader clock drops within a millisecond of idle
+    time (host work, allocations, the CPU leg) and needs tens of milliseconds of load to
+    come back; a handful of warm-up launches of a sub-millisecond kernel is not enough."""
     import torch
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    fn()
-    torch.cuda.synchronize()
-    one = max(time.perf_counter() - t0, 1e-6)
-    for _ in range(min(20000, int(ms * 1e-3 / one) + 1)):
-        fn()
-    torch.cuda.synchronize()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3
 
 

@@ -20,7 +20,11 @@
  *
  * All entry points are thread-safe and hold no state between calls.  A call may
  * issue more than one kernel on the stream.  No tensor may have 2^31 elements
- * or more (KCG_ERR_UNSUPPORTED_SHAPE).
+ * or more (KCG_ERR_UNSUPPORTED_SHAPE): the one run with a larger operand ended in a GPU
+ * memory fault whose cause is not known (a host replay of the matmul kernel's address
+ * arithmetic, tests/gemm_dl_address_model.cc, finds every access of that call inside its
+ * tensor).  The largest operand that has been run on the GPU is 1 GiB; operands between
+ * 1 GiB and the limit are accepted but unverified.
  */
 #ifndef KCG_H
 #define KCG_H
