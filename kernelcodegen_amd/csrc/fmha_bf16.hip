@@ -1041,14 +1041,17 @@ static int launch_fmha_bf16_pp(const uint16_t *Q, const uint16_t *K, const uint1
 int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, void *O,
                        int o_dtype, int B, int H, int S, int D, float scale, int causal,
                        const kcg_fmha_sched *sched, hipStream_t stream, kcg_launch_info *info) {
-  // default: 8 waves (256 query rows) share each K/V tile when the sequence is long and
-  // such workgroups (causal: pairs of them) still fill every CU; otherwise 128 rows.  On
-  // half-filled launches the small block is 30-40 % faster (B=1, H=32, S=2048 causal: 620
-  // against 476 TFLOP/s), on full ones the large block 2-6 % from S = 2048 on (D = 128) or
-  // S = 8192 on (D = 64).
+  // default, from a sweep of 38 shapes x {causal, not} x both block sizes on the box: at
+  // D = 128 the 256-row ping-pong kernel when its work items (causal: pairs of blocks) give
+  // every CU two or more, or exactly fill the CUs on a long or non-causal sweep (3-15 %
+  // faster there; on half-filled launches the 128-row block is 30-40 % faster: B=1, H=32,
+  // S=2048 causal 629 against 475 TFLOP/s).  At D = 64 a tile has half the matrix work for
+  // the same softmax, the two wave groups no longer balance, and the 128-row kernel is
+  // ahead on every shape of the sweep.
   const int64_t blocks256 = (static_cast<int64_t>(S) + 255) / 256;
   const int64_t items256 = (causal ? (blocks256 + 1) / 2 : blocks256) * B * H;
-  int br = (items256 >= kNumCu && S >= (D == 128 ? 2048 : 8192)) ? 256 : 128, bc = 64;
+  const bool large = D == 128 && (items256 >= 2 * kNumCu || (items256 >= kNumCu && (S >= 2048 || !causal)));
+  int br = large ? 256 : 128, bc = 64;
   if (sched) {
     if (sched->br) br = sched->br;
     if (sched->bc) bc = sched->bc;
