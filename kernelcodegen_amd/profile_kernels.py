@@ -26,6 +26,9 @@ def main():
                     help="a BASELINE config of the fused kernels, or an un-fused operator at the "
                          "configs[3] shape (bmmnt: Q.K^T, bmmnn: P.V, softmax: in place on the scores) "
                          "/ ReLU on a 1 GiB tensor")
+    ap.add_argument("--tile", default="",
+                    help="matmul workloads only: BLOCK_M x BLOCK_N x BLOCK_K of the schedule, e.g. 256x128x32 "
+                         "(default: the library's choice)")
     ap.add_argument("--iters", type=int, default=200,
                     help="launches of the workload (the first tens run on a ramping clock)")
     args = ap.parse_args()
@@ -63,7 +66,11 @@ def main():
         A = torch.from_numpy(c["A"]).to(dev)
         B = torch.from_numpy(c["B"]).to(dev)
         C = torch.empty((A.shape[0], B.shape[1]), dtype=torch.float32, device=dev)
-        fn = lambda: ops.matmul(A, B, relu=c["relu"], out=C)
+        sched = None
+        if args.tile:
+            bm, bn, bk = (int(x) for x in args.tile.split("x"))
+            sched = dict(block_m=bm, block_n=bn, block_k=bk)
+        fn = lambda: ops.matmul(A, B, relu=c["relu"], out=C, sched=sched)
     else:
         if c["dtype"] == "bf16":
             Q, K, V = (torch.from_numpy(c[k].view(np.int16)).to(dev).view(torch.bfloat16) for k in "QKV")
