@@ -1,7 +1,8 @@
-// Tile geometry of the direct-load matmul kernel (gemm_f32_dl_kernel): LDS layout, swizzle
-// and the split of the tile loads over waves.  Kept free of HIP headers so that a host
-// program can include it and replay the kernel's address arithmetic with the same
-// constants (tests/gemm_dl_address_model.cc does).
+// Tile geometry of the direct-load matmul kernels (gemm_f32_dl_kernel, gemm_f32_stream_kernel):
+// LDS layout, swizzle, the split of the tile loads over waves, and the streaming kernel's
+// work-item arithmetic.  Kept free of HIP headers so that a host program can include it and
+// replay the kernels' address arithmetic with the same constants and functions
+// (tests/gemm_dl_address_model.cc, tests/gemm_stream_address_model.cc).
 #pragma once
 
 #if defined(__HIPCC__)
@@ -47,5 +48,46 @@ struct GemmDlTile {
     return (k / kRowsPerRunB) * kRunB + (k % kRowsPerRunB) * BN;
   }
 };
+
+// ---- streaming kernel (gemm_f32_stream.h) ----
+struct GemmStreamGeometry {
+  static constexpr int kBM = 256, kBN = 128, kBK = 16, kWavesM = 4, kWavesN = 2;
+  static constexpr int kStages = 4;
+  static constexpr int kAhead = 3;           // slices between a load request and its use
+  static constexpr int kAccPerLane = 64;     // floats of C per lane and tile
+};
+
+// The (matrix, tile) items of workgroup `block` of a grid of `grid` workgroups: every XCD
+// (workgroup w runs on XCD w mod xcds) owns a contiguous range of the items, its
+// workgroups take them round robin: first, first + step, ... below end.
+struct GemmStreamItems {
+  int first, end, step;
+};
+KCG_HD inline GemmStreamItems gemm_stream_items(int block, int grid, int total_items, int xcds) {
+  const int xcd = block % xcds;
+  GemmStreamItems r;
+  r.step = (grid - xcd + xcds - 1) / xcds;   // workgroups on this XCD
+  r.end = static_cast<int>(static_cast<long long>(total_items) * (xcd + 1) / xcds);
+  r.first = static_cast<int>(static_cast<long long>(total_items) * xcd / xcds) + block / xcds;
+  return r;
+}
+
+// Matrix index and tile origin of an item; tiles of a matrix in group_m-wide column-major
+// groups, as in gemm_f32_dl_kernel.
+struct GemmStreamOrigin {
+  int bz, m0, n0;
+};
+KCG_HD inline GemmStreamOrigin gemm_stream_decode(int item, int tiles_m, int tiles_n, int group_m) {
+  const int per_mat = tiles_m * tiles_n;
+  const int bz = item / per_mat;
+  const int logical = item - bz * per_mat;
+  const int width = group_m * tiles_n;
+  const int group = logical / width;
+  const int first_m = group * group_m;
+  const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+  const int in_group = logical - group * width;
+  return GemmStreamOrigin{bz, (first_m + in_group % gsz) * GemmStreamGeometry::kBM,
+                          (in_group / gsz) * GemmStreamGeometry::kBN};
+}
 
 }  // namespace kcg

@@ -32,13 +32,6 @@
 
 namespace kcg {
 
-struct GemmStreamGeometry {
-  static constexpr int kBM = 256, kBN = 128, kBK = 16, kWavesM = 4, kWavesN = 2;
-  static constexpr int kStages = 4;
-  static constexpr int kAhead = 3;           // slices between a load request and its use
-  static constexpr int kAccPerLane = 64;     // floats of C per lane and tile
-};
-
 template <bool TRANS_B, int KT, bool STREAM_C>
 __global__ __launch_bounds__(512, 2) void gemm_f32_stream_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N, int K,
@@ -69,26 +62,11 @@ __global__ __launch_bounds__(512, 2) void gemm_f32_stream_kernel(
   // ---- the workgroup's list of tiles: every XCD owns a contiguous range of (matrix, tile)
   // items, its workgroups take them round robin, so that the tiles in flight on one XCD are
   // neighbours and share rows of A and B in its L2.
-  const int per_mat = tiles_m * tiles_n;
-  const int total_items = per_mat * batch;
-  const int xcd = blockIdx.x % kNumXcd;
-  const int item_step = (static_cast<int>(gridDim.x) - xcd + kNumXcd - 1) / kNumXcd;
-  const int item_end = static_cast<int>(static_cast<int64_t>(total_items) * (xcd + 1) / kNumXcd);
-  const int item_first = static_cast<int>(static_cast<int64_t>(total_items) * xcd / kNumXcd) + blockIdx.x / kNumXcd;
+  const GemmStreamItems items = gemm_stream_items(blockIdx.x, gridDim.x, tiles_m * tiles_n * batch, kNumXcd);
+  const int item_step = items.step, item_end = items.end, item_first = items.first;
   if (item_first >= item_end) return;
-  struct Origin {
-    int bz, m0, n0;
-  };
-  auto decode = [&](int item) {
-    const int bz = item / per_mat;
-    const int logical = item - bz * per_mat;
-    const int width = group_m * tiles_n;
-    const int group = logical / width;
-    const int first_m = group * group_m;
-    const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
-    const int in_group = logical - group * width;
-    return Origin{bz, (first_m + in_group % gsz) * BM, (in_group / gsz) * BN};
-  };
+  using Origin = GemmStreamOrigin;
+  auto decode = [&](int item) { return gemm_stream_decode(item, tiles_m, tiles_n, group_m); };
 
   // ---- direct loads: lane offsets are the same for every tile ----
   const int lds_base = static_cast<int>(reinterpret_cast<uintptr_t>(lds));

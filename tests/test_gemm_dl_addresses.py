@@ -1,4 +1,4 @@
-"""Address arithmetic of the direct-load matmul kernel, replayed on the host.
+"""Address arithmetic of the direct-load matmul kernels, replayed on the host.
 
 tests/gemm_dl_address_model.cc walks every workgroup, wave and lane of one launch of
 gemm_f32_dl_kernel through the kernel's own integer expressions (it shares the tile
@@ -55,5 +55,43 @@ CASES = [
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(map(str, c)))
 def test_every_access_inside_its_tensor(model, case):
     r = subprocess.run([model] + [str(v) for v in case], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert " 0 violations" in r.stdout
+
+
+# ---- the streaming kernel of BatchedMatmul (gemm_f32_stream_kernel) ----
+STREAM_SRC = os.path.join(ROOT, "tests", "gemm_stream_address_model.cc")
+
+
+@pytest.fixture(scope="module")
+def stream_model(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("gemm_stream") / "gemm_stream_address_model")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-I", INC, STREAM_SRC, "-o", exe], check=True)
+    return exe
+
+
+# (TRANS_B, BATCH, M, N, K, GRID): the attention-score product of configs[3] in both layouts,
+# the shapes of the GPU tests (item counts that 8 XCDs x 32 workgroups do not divide, K of 4,
+# 12, 20 and 64 slices), a grid smaller than the CU count, byte offsets beyond 2^32 inside C,
+# and the widest N the launcher admits (lane offsets of the stores close to 2^31).
+STREAM_CASES = [
+    (1, 32, 2048, 2048, 128, 256),
+    (0, 32, 2048, 2048, 128, 256),
+    (1, 9, 1280, 1664, 64, 256),
+    (1, 9, 1280, 1664, 192, 256),
+    (0, 20, 768, 1152, 320, 256),
+    (1, 5, 2560, 1408, 1024, 256),
+    (0, 3, 256, 384, 64, 9),
+    (1, 16, 8192, 8192, 128, 256),
+    (0, 1, 256, 2097152, 64, 256),
+]
+
+
+@pytest.mark.parametrize("case", STREAM_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_streaming_kernel_items_and_addresses(stream_model, case):
+    """Every tile is taken by exactly one workgroup, every load (the cursor that runs ahead
+    and parks on the last slice included) and every store lies inside its tensor, and the
+    stores of the eight waves cover a tile exactly once."""
+    r = subprocess.run([stream_model] + [str(v) for v in case], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout + r.stderr
     assert " 0 violations" in r.stdout
