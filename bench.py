@@ -5,7 +5,8 @@ A step is one launch of the fused fp32 matmul + ReLU kernel on BASELINE.json's
 configs[1] (M = N = K = 4096, A, B ~ N(0,1) from the seeded generator), inputs
 resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s, the roofline of the
 kernel (algorithmic FLOPs / HIP-event launch time vs the fp32 MFMA peak), the CPU
-oracle timed on the host cores, and the two attention workloads as extras.
+oracle timed on the host cores, and the two attention workloads as extras (plus the bf16
+one without its causal mask, for comparison).
 
 Every timed region is preceded by an untimed clock-settle phase (SETTLE_MS of back-to-back
 launches of the same call) in addition to the --warmup launches, so that the figures do not
@@ -247,6 +248,17 @@ def main():
                          "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(fl / (e * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
                          **traffic_fields("fmha_cfg4")}}
+        # the same tensors without the mask: what the causal structure (diagonal tiles, the
+        # restart of the second block of a pair) costs on top of the kernel's own rate
+        fl = 4.0 * Bn * H * S * S * D
+        w, e = time_launches(lambda: ops.fmha(Q, Kt, V, scale=c4["scale"], causal=False, out=O),
+                             steps, warm)
+        extras["fmha_bf16_cfg4_shape_noncausal"] = {
+            "workload": "the configs[4] tensors (bf16, B=4 H=32 S=4096 D=128) without the causal mask; not a BASELINE config",
+            "ms_per_step": round(w, 5), "value": round(fl / (w * 1e-3) / 1e12, 3), "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(fl / (e * 1e-3) / 1e12, 3),
+                         "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(fl / (e * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None}}
         out["extras"] = extras
 
     print(json.dumps(out))
