@@ -246,3 +246,35 @@ def test_python_wrappers_refuse_mismatched_tensors():
         ops.fmha(Qb, Kb, Vb, out=_meta((1, 2, 64, 32), bf16))
     with pytest.raises(ValueError):
         ops.fmha(_meta(shape, f16), _meta(shape, f16), _meta(shape, f16))
+
+
+@pytest.mark.parametrize("shape,causal,pingpong", [
+    # D = 128: the 256-row ping-pong kernel from two work items per CU on ...
+    ((4, 32, 4096, 128), 1, True),      # configs[4]: 1024 paired items
+    ((8, 32, 1024, 128), 1, True),      # 2 pairs x 256 heads = 512
+    ((32, 32, 512, 128), 1, True),      # 1 pair x 1024 heads
+    # ... or exactly filling the CUs on a long or a non-causal sweep
+    ((1, 32, 2048, 128), 0, True),      # 8 blocks x 32 heads = 256
+    ((1, 32, 4096, 128), 1, True),      # 8 pairs x 32 heads = 256, S >= 2048
+    ((4, 32, 1024, 128), 1, False),     # 256 items, short and causal: the 128-row kernel
+    ((16, 16, 512, 128), 1, False),
+    ((16, 16, 512, 128), 0, True),      # 512 items
+    # launches 256-row blocks do not fill
+    ((1, 32, 2048, 128), 1, False),
+    ((1, 16, 2048, 128), 0, False),
+    # D = 64: always the 128-row kernel
+    ((2, 16, 8192, 64), 0, False),
+    ((4, 32, 4096, 64), 1, False),
+])
+def test_bf16_attention_default_block_size(shape, causal, pingpong):
+    """The block-size rule of kcg_fmha_bf16 with no schedule given, as kcg_fmha_query reports it."""
+    L = lib.load()
+    info = lib.LaunchInfo()
+    B, H, S, D = shape
+    assert L.kcg_fmha_query(1, B, H, S, D, causal, None, ctypes.byref(info)) == 0
+    assert (b"pingpong" in info.kernel) == pingpong, info.kernel
+    assert (b"br256" in info.kernel) == pingpong
+    if pingpong:
+        blocks = (S + 255) // 256
+        items = ((blocks + 1) // 2 if causal else blocks) * B * H
+        assert info.grid[0] == min(items, 256) and info.block[0] == 512
