@@ -318,18 +318,36 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 // per tile.
 // blockIdx.y is the batch index of BatchedMatmul (src/Frontend/Operators.cc:253-420); the
 // three strides are 0 for the plain matmul.
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool RAGGED, int MIN_WAVES,
-          bool TRANS_B = false>
-__global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_dl_kernel(
+// SPLIT (full tiles only): the launch holds split_full whole tiles followed by the remaining
+// tiles cut along K into split_parts pieces, one workgroup per piece.  A piece accumulates its
+// K / split_parts slices and writes the raw 64-byte-aligned BM x BN partial tile to
+// ws[(tile - split_full) * split_parts + piece] (no epilogue); gemm_split_reduce_kernel adds
+// the pieces up.  Whole tiles run exactly as without SPLIT.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool RAGGED, bool TRANS_B, bool SPLIT>
+__device__ __forceinline__ void gemm_dl_body(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
-    int K, int tiles_m, int tiles_n, int group_m, int64_t batch_a, int64_t batch_b, int64_t batch_c) {
+    int K, int tiles_m, int tiles_n, int group_m, int64_t batch_a, int64_t batch_b, int64_t batch_c,
+    int split_full, int split_parts, float *__restrict__ ws) {
   using T = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N, TRANS_B>;
+  static_assert(!(SPLIT && (RAGGED || TRANS_B)), "K-split pieces exist for full row-major tiles only");
   extern __shared__ __align__(16) float lds[];
   A += blockIdx.y * batch_a;
   B += blockIdx.y * batch_b;
   C += blockIdx.y * batch_c;
 
-  const int logical = xcd_contiguous_id(blockIdx.x, tiles_m * tiles_n);
+  // (SPLIT: the whole tiles come first in the grid and the pieces after them, each set
+  // spread over the XCDs by itself -- split_full is a multiple of the XCD count -- so that
+  // every XCD, and every CU of it, gets the same mix)
+  int logical, piece = 0;
+  bool partial = false;
+  if (SPLIT && static_cast<int>(blockIdx.x) >= split_full) {
+    const int q = xcd_contiguous_id(blockIdx.x - split_full, static_cast<int>(gridDim.x) - split_full);
+    logical = split_full + q / split_parts;
+    piece = q - (q / split_parts) * split_parts;
+    partial = true;
+  } else {
+    logical = xcd_contiguous_id(blockIdx.x, SPLIT ? split_full : tiles_m * tiles_n);
+  }
   const int width = group_m * tiles_n;
   const int group = logical / width;
   const int first_m = group * group_m;
@@ -385,6 +403,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   const char *ga = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
   const char *gb = reinterpret_cast<const char *>(TRANS_B ? B + static_cast<int64_t>(n0) * K : B + n0);
   const int64_t b_step = TRANS_B ? BK * 4 : static_cast<int64_t>(BK) * N * 4;
+  // slices of this workgroup: all of K, or one piece of it
+  const int my_slices = (SPLIT && partial) ? (K / BK) / split_parts : K / BK;
+  if (SPLIT && partial) {
+    ga += static_cast<int64_t>(piece) * my_slices * (BK * 4);
+    gb += static_cast<int64_t>(piece) * my_slices * b_step;
+  }
   constexpr int kLoadsPerSlice = T::kInstrA + T::kInstrB;
   // load l of the slice at (ga, gb) into the stage at float offset stage_off
   auto issue_one = [&](int stage_off, int l) {
@@ -491,7 +515,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
     asm volatile("" ::: "memory");
   };
 
-  const int kfull = K / BK;                      // slices the direct loads may fetch
+  const int kfull = my_slices;                   // slices the direct loads may fetch
   const int ktiles = RAGGED ? (K + BK - 1) / BK : kfull;
   // The last, partial slice (RAGGED): rewritten through registers with zeros beyond K.
   // Lane L of load l owns the same 16 bytes of the stage as in the direct load.
@@ -637,10 +661,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   // 32-bit add per store instead of a 64-bit multiply-add -- VALU work that the short-K
   // problems (attention scores: K = 128) would otherwise pay for in matrix time.  The
   // offset stays below 2^32 because N < 2^22 on this path.
-  char *c_tile = reinterpret_cast<char *>(C + static_cast<int64_t>(m0) * N + n0);
-  const unsigned lane_off = (static_cast<unsigned>(wm * T::kWaveM + 4 * half) * static_cast<unsigned>(N) +
+  const bool to_ws = SPLIT && partial;
+  char *c_tile = to_ws ? reinterpret_cast<char *>(ws + (static_cast<int64_t>(logical - split_full) * split_parts + piece) * (BM * BN))
+                       : reinterpret_cast<char *>(C + static_cast<int64_t>(m0) * N + n0);
+  const unsigned ldc = to_ws ? static_cast<unsigned>(BN) : static_cast<unsigned>(N);
+  const unsigned lane_off = (static_cast<unsigned>(wm * T::kWaveM + 4 * half) * ldc +
                              static_cast<unsigned>(wn * T::kWaveN + r32)) * 4u;
-  const unsigned row_bytes = static_cast<unsigned>(N) * 4u;
+  const unsigned row_bytes = ldc * 4u;
   auto store_c = [&](auto stream_c) {
 #pragma unroll
     for (int i = 0; i < T::kTilesM; ++i) {
@@ -652,7 +679,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
           const int local_row = i * 32 + 8 * (e / 4) + (e % 4);
           const int row = m0 + wm * T::kWaveM + 4 * half + local_row;
           float v = acc[i][n][e];
-          if (RELU) v = relu_maxf(v);
+          if (RELU && !to_ws) v = relu_maxf(v);
           if (!RAGGED || (row < M && col < N)) {
             float *p = reinterpret_cast<float *>(c_tile + (lane_off + static_cast<unsigned>(local_row) * row_bytes +
                                                            static_cast<unsigned>(n * 32 * 4)));
@@ -665,6 +692,55 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   };
   if (static_cast<int64_t>(M) * N * gridDim.y > (int64_t{48} << 20)) store_c(std::true_type{});
   else store_c(std::false_type{});
+}
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool RAGGED, int MIN_WAVES,
+          bool TRANS_B = false>
+__global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_dl_kernel(
+    const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
+    int K, int tiles_m, int tiles_n, int group_m, int64_t batch_a, int64_t batch_b, int64_t batch_c) {
+  gemm_dl_body<BM, BN, BK, WAVES_M, WAVES_N, RELU, RAGGED, TRANS_B, false>(A, B, C, M, N, K, tiles_m, tiles_n, group_m,
+                                                                           batch_a, batch_b, batch_c, 0, 1, nullptr);
+}
+
+// The launch with K-split tail tiles (see gemm_dl_body).
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, int MIN_WAVES>
+__global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_dl_split_kernel(
+    const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
+    int K, int tiles_m, int tiles_n, int group_m, int split_full, int split_parts, float *__restrict__ ws) {
+  gemm_dl_body<BM, BN, BK, WAVES_M, WAVES_N, RELU, false, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, group_m, 0, 0,
+                                                                       0, split_full, split_parts, ws);
+}
+
+// C tile = epilogue(sum of the split_parts partial tiles), for tile split_full + blockIdx.x.
+template <int BM, int BN, bool RELU>
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *__restrict__ ws, float *__restrict__ C,
+                                                                int N, int tiles_m, int tiles_n, int group_m,
+                                                                int split_full, int split_parts) {
+  const int logical = split_full + blockIdx.x;
+  const int width = group_m * tiles_n;
+  const int group = logical / width;
+  const int first_m = group * group_m;
+  const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+  const int in_group = logical - group * width;
+  const int m0 = (first_m + in_group % gsz) * BM;
+  const int n0 = (in_group / gsz) * BN;
+  const float *src = ws + static_cast<int64_t>(blockIdx.x) * split_parts * (BM * BN);
+  constexpr int kQuads = BM * BN / 4;
+  for (int idx = threadIdx.x; idx < kQuads; idx += 256) {
+    float4_t sum = *reinterpret_cast<const float4_t *>(src + idx * 4);
+    for (int p = 1; p < split_parts; ++p) {
+      const float4_t v = *reinterpret_cast<const float4_t *>(src + static_cast<int64_t>(p) * (BM * BN) + idx * 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum[j] += v[j];
+    }
+    if (RELU) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum[j] = relu_maxf(sum[j]);
+    }
+    const int row = idx / (BN / 4), c4 = idx % (BN / 4);
+    *reinterpret_cast<float4_t *>(C + static_cast<int64_t>(m0 + row) * N + n0 + c4 * 4) = sum;
+  }
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MIN_WAVES>
@@ -909,6 +985,82 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
   return launch_sched(d, A, B, C, M, N, K, epilogue, stream, info);
 }
 
+// ---- K-split tail (the one plan that needs device memory beyond the operands) ----
+// A problem of whole 64 x 64 tiles whose tile count is a few rounds of the CUs plus a small
+// rest (1536^3: 576 = 2 x 256 + 64) holds every CU for one more round on behalf of a quarter
+// of them.  With a workspace the rest is cut along K instead: the launch holds the whole
+// tiles of the full rounds plus `parts` pieces of each remaining tile, so that every CU gets
+// the same share; the pieces go to the workspace as raw partial tiles and a second, small
+// launch adds them up and applies the epilogue.  The sums are taken in a fixed order: the
+// result does not vary from run to run (it differs from the unsplit sum in the last bits).
+struct SplitPlan {
+  int full = 0, rest = 0, parts = 0;
+  int64_t ws_bytes = 0;
+};
+static bool split_tail_plan(int64_t M, int64_t N, int64_t K, SplitPlan *out) {
+  if (M % 64 || N % 64 || K % 32 || N >= (1 << 22) || K >= (1 << 22)) return false;
+  const GemmPlan plan = default_plan(M, N);
+  if (plan.main_rows < M || plan.main.block_m != 64 || plan.main.block_n != 64) return false;
+  const int64_t tiles = (M / 64) * (N / 64);
+  const int64_t rounds = tiles / kNumCu, rest = tiles % kNumCu;
+  if (rounds < 1 || rounds > 3 || rest == 0) return false;
+  const int64_t slices = K / 32;
+  int parts = 0;
+  for (int cand : {8, 6, 4, 3, 2})
+    if (rest * cand <= kNumCu && slices % cand == 0 && slices / cand >= 4) {
+      parts = cand;
+      break;
+    }
+  // worth a second launch when the run gets at least a tenth shorter and the part of a round
+  // that is saved outweighs that launch (measured: about 8 us, the time of 750 steps of K)
+  if (parts == 0 || rounds + 1.0 / parts > 0.9 * (rounds + 1)) return false;
+  if (static_cast<double>(K) * (1.0 - 1.0 / parts) < 750.0) return false;
+  out->full = static_cast<int>(rounds * kNumCu);
+  out->rest = static_cast<int>(rest);
+  out->parts = parts;
+  out->ws_bytes = rest * parts * int64_t{64 * 64 * 4};
+  return true;
+}
+
+static int launch_split(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
+                        int group_m, const SplitPlan &sp, float *ws, hipStream_t stream) {
+  using TD = GemmDlTile<64, 64, 32, 2, 2>;
+  const int tiles_m = static_cast<int>(M / 64), tiles_n = static_cast<int>(N / 64);
+  const bool relu = epilogue == KCG_EPILOGUE_RELU;
+  const dim3 grid(static_cast<unsigned>(sp.full + sp.rest * sp.parts)), block(256);
+  auto main_launch = [&](auto kern) {
+    if (!allow_lds(kern, TD::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
+    return launch(kern, grid, block, TD::kLdsBytes, stream, A, B, C, static_cast<int>(M), static_cast<int>(N),
+                  static_cast<int>(K), tiles_m, tiles_n, group_m, sp.full, sp.parts, ws);
+  };
+  const int st = relu ? main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, true, 2>)
+                      : main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, false, 2>);
+  if (st != KCG_OK) return st;
+  const float *cws = ws;
+  return relu ? launch(gemm_split_reduce_kernel<64, 64, true>, dim3(sp.rest), dim3(256), 0, stream, cws, C,
+                       static_cast<int>(N), tiles_m, tiles_n, group_m, sp.full, sp.parts)
+              : launch(gemm_split_reduce_kernel<64, 64, false>, dim3(sp.rest), dim3(256), 0, stream, cws, C,
+                       static_cast<int>(N), tiles_m, tiles_n, group_m, sp.full, sp.parts);
+}
+
+// The schedule leaves the tile to the library (only GROUP_SIZE_M may be set).
+static bool tile_is_free(const kcg_gemm_sched *s) {
+  return !s || (s->block_m == 0 && s->block_n == 0 && s->block_k == 0 && s->wave_m == 0 && s->wave_n == 0 &&
+                s->lds_stages == 0 && (s->wave_size == 0 || s->wave_size == 64) &&
+                (s->vec_width == 0 || s->vec_width == 4));
+}
+
+// kcg_gemm_f32 with a workspace the caller lends: runs the K-split plan where there is one
+// and the workspace holds it, the plain plan otherwise.
+static int dispatch_gemm_ws(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
+                            const kcg_gemm_sched *s, float *ws, int64_t ws_bytes, hipStream_t stream) {
+  SplitPlan sp;
+  if (ws && tile_is_free(s) && split_tail_plan(M, N, K, &sp) && ws_bytes >= sp.ws_bytes && aligned16(A) &&
+      aligned16(B) && aligned16(C) && aligned16(ws))
+    return launch_split(A, B, C, M, N, K, epilogue, s && s->group_m ? s->group_m : 8, sp, ws, stream);
+  return dispatch_gemm(A, B, C, M, N, K, epilogue, s, stream, nullptr);
+}
+
 // BatchedMatmul (src/Frontend/Operators.cc:253-420) on the direct-load kernel: A row-major
 // [batch][M][K]; B [batch][K][N] or, trans_b, [batch][N][K].  Returns
 // KCG_ERR_UNSUPPORTED_SHAPE for problems this kernel does not take (rows that are not
@@ -1019,6 +1171,22 @@ int kcg_gemm_f32(const float *A, const float *B, float *C, int64_t M, int64_t N,
   if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_RELU) return KCG_ERR_BAD_ARGUMENT;
   return kcg::dispatch_gemm(A, B, C, M, N, K, epilogue, sched, static_cast<hipStream_t>(stream),
                             nullptr);
+}
+
+int64_t kcg_gemm_f32_ws_bytes(int64_t M, int64_t N, int64_t K, const kcg_gemm_sched *sched) {
+  if (gemm_shape_status(M, N, K) != KCG_OK || !kcg::tile_is_free(sched)) return 0;
+  kcg::SplitPlan sp;
+  return kcg::split_tail_plan(M, N, K, &sp) ? sp.ws_bytes : 0;
+}
+
+int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
+                    const kcg_gemm_sched *sched, void *workspace, int64_t workspace_bytes, void *stream) {
+  if (!A || !B || !C) return KCG_ERR_NULL_POINTER;
+  if (const int st = gemm_shape_status(M, N, K)) return st;
+  if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_RELU) return KCG_ERR_BAD_ARGUMENT;
+  if (workspace_bytes < 0) return KCG_ERR_BAD_ARGUMENT;
+  return kcg::dispatch_gemm_ws(A, B, C, M, N, K, epilogue, sched, static_cast<float *>(workspace), workspace_bytes,
+                               static_cast<hipStream_t>(stream));
 }
 
 int kcg_gemm_f32_query(int64_t M, int64_t N, int64_t K, const kcg_gemm_sched *sched,

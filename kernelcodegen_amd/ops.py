@@ -50,8 +50,18 @@ def _sched(sched, cls):
     return ctypes.byref(cls(**sched))
 
 
-def matmul(A, B, relu=False, out=None, sched=None):
-    """C = A.B (row-major fp32), optionally with the ReLU epilogue fused."""
+def matmul_workspace_bytes(M, N, K, sched=None):
+    """Bytes of workspace with which matmul() can run its K-split plan (0: there is none)."""
+    return int(lib.load().kcg_gemm_f32_ws_bytes(M, N, K, _sched(sched, lib.GemmSched)))
+
+
+def matmul(A, B, relu=False, out=None, sched=None, workspace=None):
+    """C = A.B (row-major fp32), optionally with the ReLU epilogue fused.
+
+    workspace: a contiguous device tensor the call may use for partial sums
+    (kcg_gemm_f32_ws; see matmul_workspace_bytes).  Nothing else may use it until the
+    call has completed on the current stream.
+    """
     _dev_f32(A, "A")
     _dev_f32(B, "B")
     M, K = A.shape
@@ -63,9 +73,17 @@ def matmul(A, B, relu=False, out=None, sched=None):
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=A.device)
     _check(out, "out", torch.float32, (M, N), A.device)
-    st = lib.load().kcg_gemm_f32(_ptr(A), _ptr(B), _ptr(out), M, N, K,
-                                 EPILOGUE_RELU if relu else EPILOGUE_NONE,
-                                 _sched(sched, lib.GemmSched), lib.current_stream())
+    epilogue = EPILOGUE_RELU if relu else EPILOGUE_NONE
+    if workspace is not None:
+        if not (isinstance(workspace, torch.Tensor) and workspace.is_cuda and workspace.device == A.device
+                and workspace.is_contiguous()):
+            raise ValueError("workspace must be a contiguous tensor on %s" % A.device)
+        st = lib.load().kcg_gemm_f32_ws(_ptr(A), _ptr(B), _ptr(out), M, N, K, epilogue,
+                                        _sched(sched, lib.GemmSched), _ptr(workspace),
+                                        workspace.numel() * workspace.element_size(), lib.current_stream())
+    else:
+        st = lib.load().kcg_gemm_f32(_ptr(A), _ptr(B), _ptr(out), M, N, K, epilogue,
+                                     _sched(sched, lib.GemmSched), lib.current_stream())
     lib.check(st)
     return out
 

@@ -268,3 +268,44 @@ def test_operands_beyond_two_to_the_31_elements(dev):
     ref2 = A2[-32:].double() @ B2.double()
     assert float((C2[-32:].double() - ref2).abs().max() / ref2.abs().max()) < TOL
 
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048)])
+def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
+    """Tile counts of whole rounds of the CUs plus a small rest (576 = 2 x 256 + 64; 272 =
+    256 + 16; 340 = 256 + 84): with a workspace the rest is cut along K (2 to 6 pieces)
+    and a second launch adds the pieces up.  Checked against the oracle, against the same
+    call without the workspace (same products, another order of summation), for equal
+    results on a second run, and for a workspace that stays inside its bytes."""
+    import torch
+    from kernelcodegen_amd import ops
+    M, N, K = shape
+    need = ops.matmul_workspace_bytes(M, N, K)
+    assert 0 < need <= 4 << 20 and need % (64 * 64 * 4) == 0
+    A = inputs.normal((M, K), 431, 0)
+    B = inputs.normal((K, N), 431, 1)
+    ref = oracle.matmul(A, B)
+    if relu:
+        ref = oracle.relu(ref)
+    tA, tB = _gpu(A, dev), _gpu(B, dev)
+    buf = torch.full((need // 4 + 256,), -7.0, device=dev)
+    C1 = ops.matmul(tA, tB, relu=relu, workspace=buf[:need // 4])
+    assert bool((buf[need // 4:] == -7.0).all())
+    assert max(rel_err(C1.cpu().numpy(), ref)) < 1e-4
+    C2 = ops.matmul(tA, tB, relu=relu, workspace=buf[:need // 4])
+    assert torch.equal(C1, C2)
+    plain = ops.matmul(tA, tB, relu=relu)
+    assert max(rel_err(C1.cpu().numpy(), plain.cpu().numpy())) < 1e-5
+    # a workspace that is too small is not used: the call is the plain one, bit for bit
+    small = ops.matmul(tA, tB, relu=relu, workspace=buf[:need // 8])
+    assert torch.equal(small, plain)
+
+
+def test_no_k_split_plan_where_it_does_not_pay(dev):
+    from kernelcodegen_amd import ops, lib
+    for shape in [(4096, 4096, 4096), (1024, 1024, 1024), (512, 512, 512), (1536, 1536, 1500), (1530, 1536, 1536),
+                  (3072, 3072, 3072), (1536, 1536, 256), (1280, 1088, 512)]:
+        assert ops.matmul_workspace_bytes(*shape) == 0, shape
+    # a fixed tile keeps its single launch
+    assert ops.matmul_workspace_bytes(1536, 1536, 1536, sched=dict(block_m=64, block_n=64, block_k=32, wave_m=32, wave_n=32)) == 0
