@@ -141,6 +141,19 @@ KCG_API int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M,
                             const kcg_gemm_sched *sched, void *workspace,
                             int64_t workspace_bytes, void *stream);
 
+/* kcg_gemm_f32_ws without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that can neither allocate device memory
+ * nor lend any: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation.  The partial sums of the K-split plan go to a 4 MiB array that is part of the
+ * library's device code (one copy per GPU, held until the process ends), which covers the
+ * largest plan; a call that needed more would return KCG_ERR_UNSUPPORTED_SHAPE.  All calls
+ * on one GPU share that array: calls that overlap in time on one GPU (two streams, two
+ * threads) race on it and must be serialised by the caller.  Same arguments, statuses and
+ * results as kcg_gemm_f32_ws with a large enough workspace. */
+KCG_API int kcg_gemm_f32_noalloc(const float *A, const float *B, float *C, int64_t M,
+                                 int64_t N, int64_t K, int epilogue,
+                                 const kcg_gemm_sched *sched, void *stream);
+
 /* ---- fused multi-head attention ------------------------------------------ */
 
 /* Schedule of the FMHA kernel: the reference's table (include/KernelCodeGen.h:

@@ -1150,6 +1150,32 @@ int dispatch_bmm_dl(const float *A, const float *B, float *C, int64_t batch, int
 
 }  // namespace kcg
 
+// ---- the partial-sum buffer of kcg_gemm_f32_noalloc ----
+// One array per GPU, part of the loaded code object: it exists from the moment the library is
+// loaded on a device until the process ends, and no call allocates or frees anything.  Every
+// call on a GPU uses that GPU's array (the K-split plan overwrites the pieces it reads, so
+// nothing has to be cleared between calls); calls that overlap in time on one GPU would
+// write each other's partial sums.
+namespace kcg_noalloc {
+constexpr int64_t kScratchBytes = int64_t{4} << 20;   // 256 partial tiles of 64 x 64 floats: the largest plan
+}
+static __device__ __align__(256) unsigned char scratch[kcg_noalloc::kScratchBytes];
+namespace kcg_noalloc {
+// Device address of `scratch` on the current device, looked up on the first call on that
+// device (in host code the array's name is only a handle for this lookup).
+static float *scratch_of_current_device() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<void *> ptrs[kMaxDevices];   // zero-initialised: not looked up yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void *p = ptrs[dev].load(std::memory_order_acquire);
+  if (p) return static_cast<float *>(p);
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+  ptrs[dev].store(p, std::memory_order_release);
+  return static_cast<float *>(p);
+}
+}  // namespace kcg_noalloc
+
 extern "C" {
 
 // Shape checks shared by the launch and the query entry point.
@@ -1186,6 +1212,21 @@ int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M, int64_t
   if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_RELU) return KCG_ERR_BAD_ARGUMENT;
   if (workspace_bytes < 0) return KCG_ERR_BAD_ARGUMENT;
   return kcg::dispatch_gemm_ws(A, B, C, M, N, K, epilogue, sched, static_cast<float *>(workspace), workspace_bytes,
+                               static_cast<hipStream_t>(stream));
+}
+
+int kcg_gemm_f32_noalloc(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
+                         const kcg_gemm_sched *sched, void *stream) {
+  if (!A || !B || !C) return KCG_ERR_NULL_POINTER;
+  if (const int st = gemm_shape_status(M, N, K)) return st;
+  if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_RELU) return KCG_ERR_BAD_ARGUMENT;
+  const int64_t need = kcg_gemm_f32_ws_bytes(M, N, K, sched);
+  if (need == 0)   // no plan with partial sums for this call: the plain one, which uses no memory of its own
+    return kcg::dispatch_gemm(A, B, C, M, N, K, epilogue, sched, static_cast<hipStream_t>(stream), nullptr);
+  if (need > kcg_noalloc::kScratchBytes) return KCG_ERR_UNSUPPORTED_SHAPE;
+  float *ws = kcg_noalloc::scratch_of_current_device();
+  if (!ws) return KCG_ERR_LAUNCH;
+  return kcg::dispatch_gemm_ws(A, B, C, M, N, K, epilogue, sched, ws, kcg_noalloc::kScratchBytes,
                                static_cast<hipStream_t>(stream));
 }
 
