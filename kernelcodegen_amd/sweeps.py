@@ -65,7 +65,7 @@ def row_bands(M):
     return [(r0, min(M, r0 + 8)) for r0 in sorted({0, max(0, M // 2 - 4), max(0, M - 8)})]
 
 
-def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None):
+def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=False):
     import numpy as np
     import torch
     from . import inputs, lib, ops
@@ -75,6 +75,8 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None):
     shapes = [(4096, 2048, 1024)] + [(d, d, d) for d in MATMUL_DIMS if d <= max_dim]
     rows = []
     _settle(dev)
+    # --workspace: the calls lend 4 MiB (kcg_gemm_f32_ws), which sizes with a K-split plan use
+    ws = torch.empty(1 << 20, dtype=torch.float32, device=dev) if workspace else None
     for (M, N, K) in shapes:
         if seeded:
             A = torch.from_numpy(inputs.uniform((M, K), MATMUL_SEED, 0)).to(dev)
@@ -90,7 +92,8 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None):
         iters = max(3, min(50, int(2e12 / flops)))
         info = lib.LaunchInfo()
         lib.check(L.kcg_gemm_f32_query(M, N, K, None, ctypes.byref(info)))
-        mine = _time(lambda: ops.matmul(A, B, relu=relu, out=C), iters)
+        mine = _time(lambda: ops.matmul(A, B, relu=relu, out=C, workspace=ws), iters)
+        split_bytes = ops.matmul_workspace_bytes(M, N, K) if workspace else 0
         if dump_dir:
             bands = np.concatenate([C[a:b].cpu().numpy() for a, b in row_bands(M)])
             np.save(os.path.join(dump_dir, "C_%dx%dx%d.npy" % (M, N, K)), bands)
@@ -110,6 +113,8 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None):
         if info.launches == 2:
             geometry += "; second launch %s on the last %d rows, grid %d x %d threads, %d B LDS" % (
                 info.tail_kernel.decode(), info.tail_rows, info.tail_grid[0], info.tail_block[0], info.tail_lds_bytes)
+        if split_bytes:
+            geometry += "; with the workspace lent: K-split plan, %d bytes of partial tiles and a second launch that adds them up" % split_bytes
         print("Matrix size : \n --- M --- : %d\n --- N --- : %d\n --- K --- : %d\n" % (M, N, K))
         print("Occupancy: %.0f%%  (computed from the launch geometry: %s, %s)" % (
             computed_occupancy_percent(info), kernels, geometry))
