@@ -8,11 +8,14 @@
 // Prints the lowest and highest byte offset reached in each tensor.  Exit status 0 = clean.
 //
 // Usage: gemm_dl_address_model BM BN BK WAVES_M WAVES_N M N K GROUP_M
+//        gemm_dl_address_model split M N K GROUP_M FULL PARTS   (the launch with K-split tail tiles)
 // Built and run by tests/test_gemm_dl_addresses.py with g++ (no GPU, no HIP).
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <initializer_list>
+#include <string>
+#include <vector>
 
 #include "gemm_dl_tile.h"
 
@@ -217,9 +220,138 @@ int replay(int64_t M64, int64_t N64, int64_t K64, int group_m) {
   return g_errors ? 1 : 0;
 }
 
+// The launch with K-split tail tiles (gemm_f32_dl_split_kernel<64, 64, 32, 2, 2> followed by
+// gemm_split_reduce_kernel): `full` whole tiles, then every remaining tile in `parts` pieces.
+// Checks the two-set numbering (every whole tile and every (tile, piece) exactly once), the K
+// range every piece loads, that the pieces fill the workspace exactly, and that whole tiles
+// plus reduced tiles write every element of C exactly once.
+int replay_split(int64_t M64, int64_t N64, int64_t K64, int group_m, int full, int parts) {
+  constexpr int BM = 64, BN = 64, BK = 32, WAVES_N = 2;
+  using T = kcg::GemmDlTile<BM, BN, BK, 2, 2, false>;
+  const int M = static_cast<int>(M64), N = static_cast<int>(N64), K = static_cast<int>(K64);
+  if (M % BM || N % BN || K % BK) return 2;
+  const int64_t bytes_a = M64 * K64 * 4, bytes_b = K64 * N64 * 4;
+  const int tiles_m = M / BM, tiles_n = N / BN, tiles = tiles_m * tiles_n;
+  const int rest = tiles - full;
+  if (full % 8 || rest <= 0 || parts < 2 || (K / BK) % parts) return 2;
+  const int grid = full + rest * parts;
+  const int64_t ws_floats = static_cast<int64_t>(rest) * parts * BM * BN;
+  std::vector<unsigned char> c_written(static_cast<size_t>(M) * N, 0), ws_written(static_cast<size_t>(ws_floats), 0);
+  std::vector<unsigned char> whole_seen(full, 0), piece_seen(static_cast<size_t>(rest) * parts, 0);
+  auto origin = [&](int logical, int *m0, int *n0) {
+    const int width = group_m * tiles_n;
+    const int group = logical / width;
+    const int first_m = group * group_m;
+    const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+    const int in_group = logical - group * width;
+    *m0 = (first_m + in_group % gsz) * BM;
+    *n0 = (in_group / gsz) * BN;
+  };
+  for (int wg = 0; wg < grid; ++wg) {
+    int logical, piece = 0;
+    bool partial = false;
+    if (wg >= full) {
+      const int q = xcd_contiguous_id(wg - full, grid - full);
+      logical = full + q / parts;
+      piece = q - (q / parts) * parts;
+      partial = true;
+      if (logical < full || logical >= tiles || piece_seen[static_cast<size_t>(logical - full) * parts + piece]++)
+        fail("piece numbering", wg, 0, 0, logical);
+    } else {
+      logical = xcd_contiguous_id(wg, full);
+      if (logical < 0 || logical >= full || whole_seen[logical]++) fail("whole tile numbering", wg, 0, 0, logical);
+    }
+    int m0, n0;
+    origin(logical, &m0, &n0);
+    if (m0 < 0 || m0 + BM > M || n0 < 0 || n0 + BN > N) fail("tile origin", wg, 0, 0, m0);
+    const int my_slices = partial ? (K / BK) / parts : K / BK;
+    const int64_t b_step = static_cast<int64_t>(BK) * N * 4;
+    const int64_t ga0 = static_cast<int64_t>(m0) * K * 4 + static_cast<int64_t>(piece) * my_slices * (BK * 4);
+    const int64_t gb0 = static_cast<int64_t>(n0) * 4 + static_cast<int64_t>(piece) * my_slices * b_step;
+    // the slice bases run from the first to the last slice of the range and then stay
+    const int64_t ga1 = ga0 + static_cast<int64_t>(my_slices - 1) * BK * 4, gb1 = gb0 + static_cast<int64_t>(my_slices - 1) * b_step;
+    // the K columns / rows this workgroup may touch
+    const int k_lo = partial ? piece * my_slices * BK : 0, k_hi = k_lo + my_slices * BK;
+    for (int wave = 0; wave < T::kWaves; ++wave) {
+      const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+      for (int lane = 0; lane < 64; ++lane) {
+        const int r32 = lane & 31, half = lane >> 5;
+        for (int i = 0; i < T::kInstrA; ++i) {
+          const int idx = (wave * T::kInstrA + i) * 256 + lane * 4;
+          const int row = idx / BK;
+          const unsigned oa = as_u32((static_cast<int64_t>(row) * K + 4 * (((idx % BK) / 4) ^ T::fa(row))) * 4, "oa", wg, wave, lane);
+          for (int64_t basep : {ga0, ga1}) {
+            const int64_t addr = basep + oa;
+            if (addr < 0 || addr + 16 > bytes_a) fail("A load out of range", wg, wave, lane, addr);
+            const int64_t col = (addr / 4) % K;
+            if (col < k_lo || col + 4 > k_hi) fail("A load outside the piece's K range", wg, wave, lane, col);
+          }
+        }
+        for (int i = 0; i < T::kInstrB; ++i) {
+          const int idx = (wave * T::kInstrB + i) * 256 + lane * 4;
+          const unsigned ob = as_u32((static_cast<int64_t>(idx / BN) * N + idx % BN) * 4, "ob", wg, wave, lane);
+          for (int64_t basep : {gb0, gb1}) {
+            const int64_t addr = basep + ob;
+            if (addr < 0 || addr + 16 > bytes_b) fail("B load out of range", wg, wave, lane, addr);
+            const int64_t krow = (addr / 4) / N;
+            if (krow < k_lo || krow >= k_hi) fail("B load outside the piece's K range", wg, wave, lane, krow);
+          }
+        }
+        // stores: to the workspace (leading dimension BN) or to C
+        const unsigned ldc = partial ? BN : static_cast<unsigned>(N);
+        const unsigned lane_off = (static_cast<unsigned>(wm * T::kWaveM + 4 * half) * ldc + static_cast<unsigned>(wn * T::kWaveN + r32)) * 4u;
+        for (int i = 0; i < T::kTilesM; ++i)
+          for (int n = 0; n < T::kTilesN; ++n)
+            for (int e = 0; e < 16; ++e) {
+              const int local_row = i * 32 + 8 * (e / 4) + (e % 4);
+              const unsigned off32 = lane_off + static_cast<unsigned>(local_row) * (ldc * 4u) + static_cast<unsigned>(n * 32 * 4);
+              if (partial) {
+                const int64_t fl = (static_cast<int64_t>(logical - full) * parts + piece) * (BM * BN) + off32 / 4;
+                if (fl < 0 || fl >= ws_floats) fail("workspace store out of range", wg, wave, lane, fl);
+                else if (ws_written[static_cast<size_t>(fl)]++) fail("workspace float written twice", wg, wave, lane, fl);
+                // position inside the partial tile = (row, column) of the tile
+                const int row = wm * T::kWaveM + 4 * half + local_row, col = wn * T::kWaveN + n * 32 + r32;
+                if (static_cast<int64_t>(off32 / 4) != static_cast<int64_t>(row) * BN + col) fail("partial tile layout", wg, wave, lane, off32);
+              } else {
+                const int64_t el = (static_cast<int64_t>(m0) * N + n0) + off32 / 4;
+                if (el < 0 || el >= static_cast<int64_t>(M) * N) fail("C store out of range", wg, wave, lane, el);
+                else if (c_written[static_cast<size_t>(el)]++) fail("C element written twice", wg, wave, lane, el);
+              }
+            }
+      }
+    }
+  }
+  // the second launch: workgroup j adds the pieces of tile full + j and writes the tile
+  for (int j = 0; j < rest; ++j) {
+    int m0, n0;
+    origin(full + j, &m0, &n0);
+    for (int idx = 0; idx < BM * BN / 4; ++idx) {
+      for (int p = 0; p < parts; ++p) {
+        const int64_t fl = (static_cast<int64_t>(j) * parts + p) * (BM * BN) + idx * 4;
+        if (fl < 0 || fl + 4 > ws_floats) fail("reduce read out of range", j, 0, 0, fl);
+      }
+      const int row = idx / (BN / 4), c4 = idx % (BN / 4);
+      for (int x = 0; x < 4; ++x) {
+        const int64_t el = static_cast<int64_t>(m0 + row) * N + n0 + c4 * 4 + x;
+        if (el < 0 || el >= static_cast<int64_t>(M) * N) fail("reduce store out of range", j, 0, 0, el);
+        else if (c_written[static_cast<size_t>(el)]++) fail("C element written twice (reduce)", j, 0, 0, el);
+      }
+    }
+  }
+  for (size_t e = 0; e < c_written.size(); ++e)
+    if (!c_written[e]) { fail("C element never written", 0, 0, 0, static_cast<int64_t>(e)); break; }
+  for (size_t e = 0; e < ws_written.size(); ++e)
+    if (!ws_written[e]) { fail("workspace float never written", 0, 0, 0, static_cast<int64_t>(e)); break; }
+  printf("split launch: %d whole tiles + %d tiles in %d pieces, grid %d, workspace %lld bytes: %d violations\n", full, rest,
+         parts, grid, static_cast<long long>(ws_floats * 4), g_errors);
+  return g_errors ? 1 : 0;
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
+  if (argc == 8 && std::string(argv[1]) == "split")
+    return replay_split(atoll(argv[2]), atoll(argv[3]), atoll(argv[4]), atoi(argv[5]), atoi(argv[6]), atoi(argv[7]));
   if (argc != 10) {
     fprintf(stderr, "usage: %s BM BN BK WAVES_M WAVES_N M N K GROUP_M\n", argv[0]);
     return 2;

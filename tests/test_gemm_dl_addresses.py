@@ -95,3 +95,24 @@ def test_streaming_kernel_items_and_addresses(stream_model, case):
     r = subprocess.run([stream_model] + [str(v) for v in case], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout + r.stderr
     assert " 0 violations" in r.stdout
+
+
+# ---- the launch with K-split tail tiles (kcg_gemm_f32_ws) ----
+@pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048),
+                                   (1536, 1536, 4096)])
+def test_k_split_launch_numbering_and_addresses(model, shape):
+    """The plan kcg_gemm_f32_ws_bytes reports (whole tiles of the full rounds, the rest in
+    pieces) replayed on the host: every whole tile and every piece is taken once, a piece
+    loads only its own K range, the pieces fill the workspace exactly, and whole tiles plus
+    reduced tiles write every element of C exactly once."""
+    from kernelcodegen_amd import lib
+    M, N, K = shape
+    need = int(lib.load().kcg_gemm_f32_ws_bytes(M, N, K, None))
+    tiles = (M // 64) * (N // 64)
+    rest = tiles % 256
+    assert need > 0 and need % (rest * 64 * 64 * 4) == 0
+    parts = need // (rest * 64 * 64 * 4)
+    r = subprocess.run([model, "split", str(M), str(N), str(K), "8", str(tiles - rest), str(parts)],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert " 0 violations" in r.stdout
