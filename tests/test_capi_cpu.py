@@ -278,3 +278,28 @@ def test_bf16_attention_default_block_size(shape, causal, pingpong):
         blocks = (S + 255) // 256
         items = ((blocks + 1) // 2 if causal else blocks) * B * H
         assert info.grid[0] == min(items, 256) and info.block[0] == 512
+
+
+def test_workspace_entry_points_check_their_arguments():
+    """kcg_gemm_f32_ws / kcg_gemm_f32_noalloc refuse what kcg_gemm_f32 refuses, before any
+    device call; kcg_gemm_f32_ws_bytes is pure host arithmetic."""
+    L = lib.load()
+    fake = ctypes.c_void_p(0x1000)
+    assert L.kcg_gemm_f32_ws(None, fake, fake, 64, 64, 64, 0, None, None, 0, None) == 1
+    assert L.kcg_gemm_f32_ws(fake, fake, fake, 64, 0, 64, 0, None, None, 0, None) == 2
+    assert L.kcg_gemm_f32_ws(fake, fake, fake, 64, 64, 64, 7, None, None, 0, None) == 5
+    assert L.kcg_gemm_f32_ws(fake, fake, fake, 64, 64, 64, 0, None, fake, -1, None) == 5
+    assert L.kcg_gemm_f32_ws(fake, fake, fake, 66000, 128, 33000, 0, None, None, 0, None) == 3
+    assert L.kcg_gemm_f32_noalloc(None, fake, fake, 64, 64, 64, 0, None, None) == 1
+    assert L.kcg_gemm_f32_noalloc(fake, fake, fake, -1, 64, 64, 0, None, None) == 2
+    assert L.kcg_gemm_f32_noalloc(fake, fake, fake, 64, 64, 64, 9, None, None) == 5
+    assert L.kcg_gemm_f32_noalloc(fake, fake, fake, 66000, 128, 33000, 0, None, None) == 3
+    # 1536^3: 576 tiles = 2 x 256 + 64, the 64 in four pieces of 64 x 64 floats
+    assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 1536, None) == 64 * 4 * 64 * 64 * 4
+    assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 256, None) == 0       # too little K to pay for a second launch
+    assert L.kcg_gemm_f32_ws_bytes(4096, 4096, 4096, None) == 0      # the large tile, evenly filled
+    assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 1540, None) == 0      # not whole slices
+    assert L.kcg_gemm_f32_ws_bytes(0, 1536, 1536, None) == 0
+    fixed = lib.GemmSched(block_m=64, block_n=64, block_k=32, wave_m=32, wave_n=32)
+    assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 1536, ctypes.byref(fixed)) == 0
+    assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 1536, ctypes.byref(lib.GemmSched(group_m=4))) == 64 * 4 * 64 * 64 * 4
