@@ -1003,7 +1003,7 @@ static bool split_tail_plan(int64_t M, int64_t N, int64_t K, SplitPlan *out) {
   if (plan.main_rows < M || plan.main.block_m != 64 || plan.main.block_n != 64) return false;
   const int64_t tiles = (M / 64) * (N / 64);
   const int64_t rounds = tiles / kNumCu, rest = tiles % kNumCu;
-  if (rounds < 1 || rounds > 3 || rest == 0) return false;
+  if (rounds > 3 || rest == 0) return false;
   const int64_t slices = K / 32;
   int parts = 0;
   for (int cand : {8, 6, 4, 3, 2})

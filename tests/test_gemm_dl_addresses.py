@@ -99,7 +99,7 @@ def test_streaming_kernel_items_and_addresses(stream_model, case):
 
 # ---- the launch with K-split tail tiles (kcg_gemm_f32_ws) ----
 @pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048),
-                                   (1536, 1536, 4096)])
+                                   (1536, 1536, 4096), (512, 512, 4096), (256, 256, 8192), (512, 1024, 2048)])
 def test_k_split_launch_numbering_and_addresses(model, shape):
     """The plan kcg_gemm_f32_ws_bytes reports (whole tiles of the full rounds, the rest in
     pieces) replayed on the host: every whole tile and every piece is taken once, a piece

@@ -271,10 +271,12 @@ def test_operands_beyond_two_to_the_31_elements(dev):
 
 
 @pytest.mark.parametrize("relu", [False, True])
-@pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048)])
+@pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048),
+                                   (512, 512, 4096), (256, 256, 8192), (512, 1024, 2048)])
 def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
     """Tile counts of whole rounds of the CUs plus a small rest (576 = 2 x 256 + 64; 272 =
-    256 + 16; 340 = 256 + 84): with a workspace the rest is cut along K (2 to 6 pieces)
+    256 + 16; 340 = 256 + 84), and problems with a long K and fewer tiles than CUs (64, 16,
+    128 tiles: every tile is cut): with a workspace the rest is cut along K (2 to 8 pieces)
     and a second launch adds the pieces up.  Checked against the oracle, against the same
     call without the workspace (same products, another order of summation), for equal
     results on a second run, and for a workspace that stays inside its bytes."""
@@ -296,7 +298,7 @@ def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
     C2 = ops.matmul(tA, tB, relu=relu, workspace=buf[:need // 4])
     assert torch.equal(C1, C2)
     plain = ops.matmul(tA, tB, relu=relu)
-    assert max(rel_err(C1.cpu().numpy(), plain.cpu().numpy())) < 1e-5
+    assert max(rel_err(C1.cpu().numpy(), plain.cpu().numpy())) < 5e-5
     # a workspace that is too small is not used: the call is the plain one, bit for bit
     small = ops.matmul(tA, tB, relu=relu, workspace=buf[:need // 8])
     assert torch.equal(small, plain)
