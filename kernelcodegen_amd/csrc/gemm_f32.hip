@@ -712,12 +712,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
                                                                        0, split_full, split_parts, ws);
 }
 
-// C tile = epilogue(sum of the split_parts partial tiles), for tile split_full + blockIdx.x.
+// C tile = epilogue(sum of the split_parts partial tiles).  A tile is shared by
+// kSplitReduceSlabs workgroups (one float4 per thread each), so that the launch spreads over
+// the chip; a thread requests its float4 of every piece before the first add (pieces beyond
+// split_parts re-read piece 0 and are left out of the sum) and adds them in piece order.
+constexpr int kSplitMaxParts = 8;
+template <int BM, int BN>
+constexpr int kSplitReduceSlabs = BM * BN / 4 / 256;
 template <int BM, int BN, bool RELU>
 __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *__restrict__ ws, float *__restrict__ C,
                                                                 int N, int tiles_m, int tiles_n, int group_m,
                                                                 int split_full, int split_parts) {
-  const int logical = split_full + blockIdx.x;
+  constexpr int kSlabs = kSplitReduceSlabs<BM, BN>;
+  static_assert(kSlabs * 256 * 4 == BM * BN, "one float4 per thread");
+  const int tile = blockIdx.x / kSlabs, slab = blockIdx.x % kSlabs;
+  const int logical = split_full + tile;
   const int width = group_m * tiles_n;
   const int group = logical / width;
   const int first_m = group * group_m;
@@ -725,22 +734,25 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *__r
   const int in_group = logical - group * width;
   const int m0 = (first_m + in_group % gsz) * BM;
   const int n0 = (in_group / gsz) * BN;
-  const float *src = ws + static_cast<int64_t>(blockIdx.x) * split_parts * (BM * BN);
-  constexpr int kQuads = BM * BN / 4;
-  for (int idx = threadIdx.x; idx < kQuads; idx += 256) {
-    float4_t sum = *reinterpret_cast<const float4_t *>(src + idx * 4);
-    for (int p = 1; p < split_parts; ++p) {
-      const float4_t v = *reinterpret_cast<const float4_t *>(src + static_cast<int64_t>(p) * (BM * BN) + idx * 4);
+  const int idx = slab * 256 + threadIdx.x;
+  const float *src = ws + static_cast<int64_t>(tile) * split_parts * (BM * BN) + idx * 4;
+  float4_t v[kSplitMaxParts];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) sum[j] += v[j];
-    }
-    if (RELU) {
+  for (int p = 0; p < kSplitMaxParts; ++p)
+    v[p] = *reinterpret_cast<const float4_t *>(src + (p < split_parts ? p : 0) * (BM * BN));
+  float4_t sum = v[0];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) sum[j] = relu_maxf(sum[j]);
+  for (int p = 1; p < kSplitMaxParts; ++p)
+    if (p < split_parts) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum[j] += v[p][j];
     }
-    const int row = idx / (BN / 4), c4 = idx % (BN / 4);
-    *reinterpret_cast<float4_t *>(C + static_cast<int64_t>(m0 + row) * N + n0 + c4 * 4) = sum;
+  if (RELU) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sum[j] = relu_maxf(sum[j]);
   }
+  const int row = idx / (BN / 4), c4 = idx % (BN / 4);
+  *reinterpret_cast<float4_t *>(C + static_cast<int64_t>(m0 + row) * N + n0 + c4 * 4) = sum;
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MIN_WAVES>
@@ -1006,6 +1018,7 @@ static bool split_tail_plan(int64_t M, int64_t N, int64_t K, SplitPlan *out) {
   if (rounds > 3 || rest == 0) return false;
   const int64_t slices = K / 32;
   int parts = 0;
+  static_assert(kSplitMaxParts == 8, "the candidates below");
   for (int cand : {8, 6, 4, 3, 2})
     if (rest * cand <= kNumCu && slices % cand == 0 && slices / cand >= 4) {
       parts = cand;
@@ -1037,9 +1050,10 @@ static int launch_split(const float *A, const float *B, float *C, int64_t M, int
                       : main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, false, 2>);
   if (st != KCG_OK) return st;
   const float *cws = ws;
-  return relu ? launch(gemm_split_reduce_kernel<64, 64, true>, dim3(sp.rest), dim3(256), 0, stream, cws, C,
+  const dim3 reduce_grid(static_cast<unsigned>(sp.rest * kSplitReduceSlabs<64, 64>));
+  return relu ? launch(gemm_split_reduce_kernel<64, 64, true>, reduce_grid, dim3(256), 0, stream, cws, C,
                        static_cast<int>(N), tiles_m, tiles_n, group_m, sp.full, sp.parts)
-              : launch(gemm_split_reduce_kernel<64, 64, false>, dim3(sp.rest), dim3(256), 0, stream, cws, C,
+              : launch(gemm_split_reduce_kernel<64, 64, false>, reduce_grid, dim3(256), 0, stream, cws, C,
                        static_cast<int>(N), tiles_m, tiles_n, group_m, sp.full, sp.parts);
 }
 

@@ -22,10 +22,11 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="gemm_cfg1",
                     choices=["gemm_cfg0", "gemm_cfg1", "gemm_cfg2", "fmha_cfg3", "fmha_cfg4",
-                             "bmmnt_cfg3", "bmmnn_cfg3", "softmax_cfg3", "relu_1gib"],
+                             "bmmnt_cfg3", "bmmnn_cfg3", "softmax_cfg3", "relu_1gib", "gemm_ksplit"],
                     help="a BASELINE config of the fused kernels, or an un-fused operator at the "
                          "configs[3] shape (bmmnt: Q.K^T, bmmnn: P.V, softmax: in place on the scores) "
-                         "/ ReLU on a 1 GiB tensor")
+                         "/ ReLU on a 1 GiB tensor / gemm_ksplit: 1536^3 (+ReLU) through the workspace entry "
+                         "point, whose plan is two launches (whole tiles and K pieces, then the sum of the pieces)")
     ap.add_argument("--tile", default="",
                     help="matmul workloads only: BLOCK_M x BLOCK_N x BLOCK_K of the schedule, e.g. 256x128x32 "
                          "(default: the library's choice)")
@@ -62,6 +63,14 @@ def main():
         else:
             P.mul_(c["scale"])
             fn = lambda: ops.softmax_(P)
+    elif args.workload == "gemm_ksplit":
+        d = 1536
+        A = torch.empty(d, d, device=dev).normal_()
+        B = torch.empty(d, d, device=dev).normal_()
+        C = torch.empty(d, d, device=dev)
+        ws = torch.empty(ops.matmul_workspace_bytes(d, d, d) // 4, dtype=torch.float32, device=dev)
+        assert ws.numel() > 0
+        fn = lambda: ops.matmul(A, B, relu=True, out=C, workspace=ws)
     elif kind == "gemm":
         A = torch.from_numpy(c["A"]).to(dev)
         B = torch.from_numpy(c["B"]).to(dev)

@@ -321,13 +321,17 @@ int replay_split(int64_t M64, int64_t N64, int64_t K64, int group_m, int full, i
       }
     }
   }
-  // the second launch: workgroup j adds the pieces of tile full + j and writes the tile
-  for (int j = 0; j < rest; ++j) {
+  // the second launch: four workgroups per remaining tile, one float4 per thread; a thread
+  // reads its float4 of all eight piece slots (slots beyond `parts` re-read piece 0)
+  constexpr int kSlabs = BM * BN / 4 / 256;
+  for (int wg = 0; wg < rest * kSlabs; ++wg) {
+    const int j = wg / kSlabs, slab = wg % kSlabs;
     int m0, n0;
     origin(full + j, &m0, &n0);
-    for (int idx = 0; idx < BM * BN / 4; ++idx) {
-      for (int p = 0; p < parts; ++p) {
-        const int64_t fl = (static_cast<int64_t>(j) * parts + p) * (BM * BN) + idx * 4;
+    for (int tid = 0; tid < 256; ++tid) {
+      const int idx = slab * 256 + tid;
+      for (int p = 0; p < 8; ++p) {
+        const int64_t fl = static_cast<int64_t>(j) * parts * (BM * BN) + idx * 4 + static_cast<int64_t>(p < parts ? p : 0) * (BM * BN);
         if (fl < 0 || fl + 4 > ws_floats) fail("reduce read out of range", j, 0, 0, fl);
       }
       const int row = idx / (BN / 4), c4 = idx % (BN / 4);
