@@ -128,14 +128,16 @@ KCG_API int kcg_gemm_f32_query(int64_t M, int64_t N, int64_t K,
  * takes A, B, C only (src/Backend/CUDA.cc:793-801) and every plan of kcg_gemm_f32 keeps to
  * that; one more plan needs device memory for partial sums: where the problem consists of
  * whole 64 x 64 tiles, the tile is left to the library, K is long enough to pay for a second
- * launch and the tile count is a few rounds of the compute units plus a small rest
- * (1536^3), or smaller than the number of compute units altogether (512 x 512 x 4096), the
- * rest is cut along K and the pieces are added up by a second launch (fixed order: results
- * do not vary between runs).
- * kcg_gemm_f32_ws_bytes gives the bytes that plan needs, 0 where there is none (at most
- * 4 MiB).  `workspace` must be 16-byte aligned device memory of at least that many bytes
- * which nothing else uses until the call has completed on `stream`; with NULL or less the
- * call behaves exactly like kcg_gemm_f32.  Same arguments and statuses otherwise. */
+ * launch and the tile count is a few rounds of the compute units plus a rest (1536^3:
+ * 2 x 256 + 64), or smaller than the number of compute units altogether (512 x 512 x 4096),
+ * the tiles of the rest are cut along K into 2 to 8 pieces each and the pieces are added up
+ * by a second launch (fixed order: results do not vary between runs).
+ * kcg_gemm_f32_ws_bytes gives the bytes the preferred plan needs, 0 where there is none (at
+ * most 32 MiB).  `workspace` must be 16-byte aligned device memory which nothing else uses
+ * until the call has completed on `stream`; the call runs the best plan whose partial sums
+ * fit into `workspace_bytes` (fewer pieces per tile than the preferred plan, if need be) and,
+ * with NULL or where none fits, behaves exactly like kcg_gemm_f32.  Same arguments and
+ * statuses otherwise. */
 KCG_API int64_t kcg_gemm_f32_ws_bytes(int64_t M, int64_t N, int64_t K,
                                       const kcg_gemm_sched *sched);
 KCG_API int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M,
@@ -147,11 +149,12 @@ KCG_API int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M,
  * counterpart in the reference; it is for callers that can neither allocate device memory
  * nor lend any: code under HIP graph capture, tight serving loops, harnesses that forbid
  * allocation.  The partial sums of the K-split plan go to a 4 MiB array that is part of the
- * library's device code (one copy per GPU, held until the process ends), which covers the
- * largest plan; a call that needed more would return KCG_ERR_UNSUPPORTED_SHAPE.  All calls
- * on one GPU share that array: calls that overlap in time on one GPU (two streams, two
- * threads) race on it and must be serialised by the caller.  Same arguments, statuses and
- * results as kcg_gemm_f32_ws with a large enough workspace. */
+ * library's device code (one copy per GPU, held until the process ends): the call runs the
+ * plan kcg_gemm_f32_ws runs when it is lent exactly 4 MiB (256 pieces at most; plans with
+ * more pieces are not considered, a plan that did not fit would be refused with
+ * KCG_ERR_UNSUPPORTED_SHAPE).  All calls on one GPU share that array: calls that overlap in
+ * time on one GPU (two streams, two threads) race on it and must be serialised by the
+ * caller.  Same arguments, statuses and results as kcg_gemm_f32_ws with 4 MiB. */
 KCG_API int kcg_gemm_f32_noalloc(const float *A, const float *B, float *C, int64_t M,
                                  int64_t N, int64_t K, int epilogue,
                                  const kcg_gemm_sched *sched, void *stream);

@@ -1009,7 +1009,13 @@ struct SplitPlan {
   int full = 0, rest = 0, parts = 0;
   int64_t ws_bytes = 0;
 };
-static bool split_tail_plan(int64_t M, int64_t N, int64_t K, SplitPlan *out) {
+// Picks the number of pieces per remaining tile.  Times in steps of K of one 64 x 64 tile: a
+// whole tile costs K, a piece K / parts plus a fixed part (its prologue and its 16 KiB of
+// partial sums, measured at about 100 steps); pieces beyond one per CU run as further waves
+// of pieces.  `max_bytes` bounds the workspace the plan may need.
+constexpr int64_t kSplitPieceBytes = 64 * 64 * 4;
+constexpr int64_t kSplitMaxPieces = 2048;   // 32 MiB of partial sums at most
+static bool split_tail_plan(int64_t M, int64_t N, int64_t K, int64_t max_bytes, SplitPlan *out) {
   if (M % 64 || N % 64 || K % 32 || N >= (1 << 22) || K >= (1 << 22)) return false;
   const GemmPlan plan = default_plan(M, N);
   if (plan.main_rows < M || plan.main.block_m != 64 || plan.main.block_n != 64) return false;
@@ -1017,21 +1023,29 @@ static bool split_tail_plan(int64_t M, int64_t N, int64_t K, SplitPlan *out) {
   const int64_t rounds = tiles / kNumCu, rest = tiles % kNumCu;
   if (rounds > 3 || rest == 0) return false;
   const int64_t slices = K / 32;
+  const int64_t max_pieces = std::min(max_bytes / kSplitPieceBytes, kSplitMaxPieces);
+  constexpr double kPieceOverhead = 100.0;
+  const double plain = static_cast<double>(rounds + 1) * K;
+  double best = plain;
   int parts = 0;
   static_assert(kSplitMaxParts == 8, "the candidates below");
-  for (int cand : {8, 6, 4, 3, 2})
-    if (rest * cand <= kNumCu && slices % cand == 0 && slices / cand >= 4) {
+  for (int cand : {2, 3, 4, 5, 6, 8}) {
+    if (slices % cand != 0 || slices / cand < 4 || rest * cand > max_pieces) continue;
+    const int64_t waves = (rest * cand + kNumCu - 1) / kNumCu;
+    const double cost = static_cast<double>(rounds) * K + waves * (static_cast<double>(K) / cand + kPieceOverhead);
+    if (cost < best) {
+      best = cost;
       parts = cand;
-      break;
     }
-  // worth a second launch when the run gets at least a tenth shorter and the part of a round
-  // that is saved outweighs that launch (measured: about 8 us, the time of 750 steps of K)
-  if (parts == 0 || rounds + 1.0 / parts > 0.9 * (rounds + 1)) return false;
-  if (static_cast<double>(K) * (1.0 - 1.0 / parts) < 750.0) return false;
+  }
+  // worth a second launch when the model's saving outweighs that launch; the bounds are
+  // measured ones (768 x 768 x 1536 at 312 steps saved still gains 10 %, 1536 x 1536 x 512 at
+  // 284 loses; 1344 x 1344 x 4096 at 5 % of the run gains 4 %)
+  if (parts == 0 || best > 0.95 * plain || plain - best < 300.0) return false;
   out->full = static_cast<int>(rounds * kNumCu);
   out->rest = static_cast<int>(rest);
   out->parts = parts;
-  out->ws_bytes = rest * parts * int64_t{64 * 64 * 4};
+  out->ws_bytes = rest * parts * kSplitPieceBytes;
   return true;
 }
 
@@ -1069,7 +1083,7 @@ static bool tile_is_free(const kcg_gemm_sched *s) {
 static int dispatch_gemm_ws(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
                             const kcg_gemm_sched *s, float *ws, int64_t ws_bytes, hipStream_t stream) {
   SplitPlan sp;
-  if (ws && tile_is_free(s) && split_tail_plan(M, N, K, &sp) && ws_bytes >= sp.ws_bytes && aligned16(A) &&
+  if (ws && tile_is_free(s) && split_tail_plan(M, N, K, ws_bytes, &sp) && aligned16(A) &&
       aligned16(B) && aligned16(C) && aligned16(ws))
     return launch_split(A, B, C, M, N, K, epilogue, s && s->group_m ? s->group_m : 8, sp, ws, stream);
   return dispatch_gemm(A, B, C, M, N, K, epilogue, s, stream, nullptr);
@@ -1216,7 +1230,7 @@ int kcg_gemm_f32(const float *A, const float *B, float *C, int64_t M, int64_t N,
 int64_t kcg_gemm_f32_ws_bytes(int64_t M, int64_t N, int64_t K, const kcg_gemm_sched *sched) {
   if (gemm_shape_status(M, N, K) != KCG_OK || !kcg::tile_is_free(sched)) return 0;
   kcg::SplitPlan sp;
-  return kcg::split_tail_plan(M, N, K, &sp) ? sp.ws_bytes : 0;
+  return kcg::split_tail_plan(M, N, K, INT64_MAX, &sp) ? sp.ws_bytes : 0;
 }
 
 int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
@@ -1234,10 +1248,12 @@ int kcg_gemm_f32_noalloc(const float *A, const float *B, float *C, int64_t M, in
   if (!A || !B || !C) return KCG_ERR_NULL_POINTER;
   if (const int st = gemm_shape_status(M, N, K)) return st;
   if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_RELU) return KCG_ERR_BAD_ARGUMENT;
-  const int64_t need = kcg_gemm_f32_ws_bytes(M, N, K, sched);
-  if (need == 0)   // no plan with partial sums for this call: the plain one, which uses no memory of its own
+  // the plan is looked for among those whose partial sums fit the array; where there is none
+  // the call is the plain one, which uses no memory of its own
+  kcg::SplitPlan sp;
+  if (!kcg::tile_is_free(sched) || !kcg::split_tail_plan(M, N, K, kcg_noalloc::kScratchBytes, &sp))
     return kcg::dispatch_gemm(A, B, C, M, N, K, epilogue, sched, static_cast<hipStream_t>(stream), nullptr);
-  if (need > kcg_noalloc::kScratchBytes) return KCG_ERR_UNSUPPORTED_SHAPE;
+  if (sp.ws_bytes > kcg_noalloc::kScratchBytes) return KCG_ERR_UNSUPPORTED_SHAPE;
   float *ws = kcg_noalloc::scratch_of_current_device();
   if (!ws) return KCG_ERR_LAUNCH;
   return kcg::dispatch_gemm_ws(A, B, C, M, N, K, epilogue, sched, ws, kcg_noalloc::kScratchBytes,

@@ -272,19 +272,21 @@ def test_operands_beyond_two_to_the_31_elements(dev):
 
 @pytest.mark.parametrize("relu", [False, True])
 @pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048),
-                                   (512, 512, 4096), (256, 256, 8192), (512, 1024, 2048)])
+                                   (512, 512, 4096), (256, 256, 8192), (512, 1024, 2048), (768, 768, 3072),
+                                   (1280, 1280, 4096)])
 def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
     """Tile counts of whole rounds of the CUs plus a small rest (576 = 2 x 256 + 64; 272 =
     256 + 16; 340 = 256 + 84), and problems with a long K and fewer tiles than CUs (64, 16,
-    128 tiles: every tile is cut): with a workspace the rest is cut along K (2 to 8 pieces)
-    and a second launch adds the pieces up.  Checked against the oracle, against the same
+    128, 144 tiles: every tile is cut; 400 = 256 + 144 in eight pieces each: more pieces than
+    CUs): with a workspace the rest is cut along K (2 to 8 pieces) and a second launch adds
+    the pieces up.  Checked against the oracle, against the same
     call without the workspace (same products, another order of summation), for equal
     results on a second run, and for a workspace that stays inside its bytes."""
     import torch
     from kernelcodegen_amd import ops
     M, N, K = shape
     need = ops.matmul_workspace_bytes(M, N, K)
-    assert 0 < need <= 4 << 20 and need % (64 * 64 * 4) == 0
+    assert 0 < need <= 32 << 20 and need % (64 * 64 * 4) == 0
     A = inputs.normal((M, K), 431, 0)
     B = inputs.normal((K, N), 431, 1)
     ref = oracle.matmul(A, B)
@@ -299,9 +301,18 @@ def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
     assert torch.equal(C1, C2)
     plain = ops.matmul(tA, tB, relu=relu)
     assert max(rel_err(C1.cpu().numpy(), plain.cpu().numpy())) < 5e-5
-    # a workspace that is too small is not used: the call is the plain one, bit for bit
-    small = ops.matmul(tA, tB, relu=relu, workspace=buf[:need // 8])
+    # a workspace too small for any plan is not used: the call is the plain one, bit for bit
+    assert need // 8 < (M // 64) * (N // 64) % 256 * 2 * 64 * 64 * 4   # not even two pieces per tile
+    small = ops.matmul(tA, tB, relu=relu, workspace=buf[:need // 8 // 4])
     assert torch.equal(small, plain)
+    if shape == (1280, 1088, 2048):
+        # 4 MiB do not hold the eight pieces per tile of the preferred plan, but two per tile
+        assert need > 4 << 20
+        buf.fill_(-7.0)
+        C3 = ops.matmul(tA, tB, relu=relu, workspace=buf[:1 << 20])
+        assert bool((buf[84 * 2 * 64 * 64:] == -7.0).all()) and not bool((buf[:84 * 2 * 64 * 64] == -7.0).any())
+        assert max(rel_err(C3.cpu().numpy(), ref)) < 1e-4
+        assert not torch.equal(C3, plain)
 
 
 def test_no_k_split_plan_where_it_does_not_pay(dev):

@@ -1,9 +1,11 @@
 """kcg_gemm_f32_noalloc: the K-split matmul plan with its partial sums in the library's own
 static device array, against kcg_gemm_f32_ws with a workspace lent by the caller.
 
-Both entry points run the same two kernels on the same operands, so their results must be
-equal bit for bit; the oracle bounds both.  Two calls in a row, the second on a smaller
-problem (fewer and other pieces in the same array), then a problem without a K-split plan.
+Lent the 4 MiB the static array has, the workspace entry point picks the same plan and runs
+the same two kernels on the same operands, so the results must be equal bit for bit; the
+oracle bounds both.  Calls in a row on smaller problems (fewer and other pieces in the same
+array): one whose preferred plan would need 10.5 MiB and runs with two pieces per tile
+instead of eight, then one without a K-split plan.
 """
 import ctypes
 
@@ -27,7 +29,9 @@ def test_noalloc_entry_point_matches_the_workspace_entry_point(oracle, dev):
     L = lib.load()
     stream = lib.current_stream()
     vp = ctypes.c_void_p
-    for seed, (M, N, K), relu in [(451, (1536, 1536, 1536), 1), (452, (1024, 1088, 1536), 0), (453, (512, 512, 512), 1)]:
+    array_bytes = 4 << 20
+    for seed, (M, N, K), relu in [(451, (1536, 1536, 1536), 1), (452, (1024, 1088, 1536), 0),
+                                  (454, (1280, 1088, 2048), 1), (453, (512, 512, 512), 1)]:
         A = inputs.normal((M, K), seed, 0)
         B = inputs.normal((K, N), seed, 1)
         ref = oracle.matmul(A, B)
@@ -35,12 +39,12 @@ def test_noalloc_entry_point_matches_the_workspace_entry_point(oracle, dev):
             ref = oracle.relu(ref)
         tA, tB = _gpu(A, dev), _gpu(B, dev)
         need = int(L.kcg_gemm_f32_ws_bytes(M, N, K, None))
-        assert (need > 0) == (K == 1536)
-        ws = torch.empty(max(need, 16) // 4, dtype=torch.float32, device=dev)
+        assert (need > 0) == (K != 512) and (need > array_bytes) == (K == 2048)
+        ws = torch.empty(array_bytes // 4, dtype=torch.float32, device=dev)
         C_ws = torch.full((M, N), -3.0, dtype=torch.float32, device=dev)
         C_na = torch.full((M, N), -5.0, dtype=torch.float32, device=dev)
         assert L.kcg_gemm_f32_ws(vp(tA.data_ptr()), vp(tB.data_ptr()), vp(C_ws.data_ptr()), M, N, K, relu, None,
-                                 vp(ws.data_ptr()), need, stream) == 0
+                                 vp(ws.data_ptr()), array_bytes, stream) == 0
         assert L.kcg_gemm_f32_noalloc(vp(tA.data_ptr()), vp(tB.data_ptr()), vp(C_na.data_ptr()), M, N, K, relu, None,
                                       stream) == 0
         torch.cuda.synchronize()
