@@ -884,7 +884,7 @@ struct GemmPlan {
   int64_t main_rows;
   kcg_gemm_sched tail;
 };
-static GemmPlan default_plan(int64_t M, int64_t N) {
+static GemmPlan default_plan(int64_t M, int64_t N, double *cost_out = nullptr) {
   GemmPlan plan;
   double single = 0.0;
   plan.main = default_tile(M, N, 1, &single);
@@ -899,6 +899,7 @@ static GemmPlan default_plan(int64_t M, int64_t N) {
   const int64_t tiles = rows_of_tiles * ((N + big.bn - 1) / big.bn);
   const int64_t spill = tiles % kNumCu;
   const int64_t max_spill = tiles >= 10 * kNumCu ? kNumCu * 11 / 20 : kNumCu * 7 / 20;
+  if (cost_out) *cost_out = single;
   if (tiles <= kNumCu || spill == 0 || spill > max_spill) return plan;
   double best = single;
   for (int64_t k = 1; k <= 8 && k < rows_of_tiles; ++k) {
@@ -914,6 +915,7 @@ static GemmPlan default_plan(int64_t M, int64_t N) {
       plan.tail = t;
     }
   }
+  if (cost_out) *cost_out = best;
   return plan;
 }
 
@@ -1012,20 +1014,26 @@ struct SplitPlan {
 // Picks the number of pieces per remaining tile.  Times in steps of K of one 64 x 64 tile: a
 // whole tile costs K, a piece K / parts plus a fixed part (its prologue and its 16 KiB of
 // partial sums, measured at about 100 steps); pieces beyond one per CU run as further waves
-// of pieces.  `max_bytes` bounds the workspace the plan may need.
+// of pieces.  The plan competes with the default plan of kcg_gemm_f32 (any tile, one launch
+// or two), priced by the same model as default_tile.  `max_bytes` bounds the workspace the
+// plan may need.
 constexpr int64_t kSplitPieceBytes = 64 * 64 * 4;
 constexpr int64_t kSplitMaxPieces = 2048;   // 32 MiB of partial sums at most
 static bool split_tail_plan(int64_t M, int64_t N, int64_t K, int64_t max_bytes, SplitPlan *out) {
   if (M % 64 || N % 64 || K % 32 || N >= (1 << 22) || K >= (1 << 22)) return false;
-  const GemmPlan plan = default_plan(M, N);
-  if (plan.main_rows < M || plan.main.block_m != 64 || plan.main.block_n != 64) return false;
+  const TileCand &small = kTileCands[3];
+  static_assert(kTileCands[3].bm == 64 && kTileCands[3].bn == 64 && kTileCands[3].bk == 32, "the tile of the split kernel");
   const int64_t tiles = (M / 64) * (N / 64);
+  if (static_cast<double>(tiles) > small.max_tiles) return false;
   const int64_t rounds = tiles / kNumCu, rest = tiles % kNumCu;
-  if (rounds > 3 || rest == 0) return false;
+  if (rest == 0) return false;
+  // the default plan in steps of K of a 64 x 64 tile at that tile's efficiency
+  double default_area = 0.0;
+  default_plan(M, N, &default_area);
+  const double plain = default_area * small.eff / (64.0 * 64.0) * K;
   const int64_t slices = K / 32;
   const int64_t max_pieces = std::min(max_bytes / kSplitPieceBytes, kSplitMaxPieces);
   constexpr double kPieceOverhead = 100.0;
-  const double plain = static_cast<double>(rounds + 1) * K;
   double best = plain;
   int parts = 0;
   static_assert(kSplitMaxParts == 8, "the candidates below");
@@ -1040,8 +1048,11 @@ static bool split_tail_plan(int64_t M, int64_t N, int64_t K, int64_t max_bytes, 
   }
   // worth a second launch when the model's saving outweighs that launch; the bounds are
   // measured ones (768 x 768 x 1536 at 312 steps saved still gains 10 %, 1536 x 1536 x 512 at
-  // 284 loses; 1344 x 1344 x 4096 at 5 % of the run gains 4 %)
-  if (parts == 0 || best > 0.95 * plain || plain - best < 300.0) return false;
+  // 284 loses; 1344 x 1344 x 4096 at 5 % of the run gains 4 %).  The first launch must also
+  // run long enough for the second to be queued behind it: calls shorter than that are
+  // bound by the host's launch rate, and two launches take twice as long as one
+  // (512 x 512 x 768, 292 steps: 5 % slower; 512 x 512 x 1024, 356 steps: 30 % faster).
+  if (parts == 0 || best > 0.95 * plain || plain - best < 300.0 || best < 330.0) return false;
   out->full = static_cast<int>(rounds * kNumCu);
   out->rest = static_cast<int>(rest);
   out->parts = parts;

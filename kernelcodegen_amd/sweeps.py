@@ -65,7 +65,7 @@ def row_bands(M):
     return [(r0, min(M, r0 + 8)) for r0 in sorted({0, max(0, M // 2 - 4), max(0, M - 8)})]
 
 
-def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=False):
+def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=False, dims=None):
     import numpy as np
     import torch
     from . import inputs, lib, ops
@@ -73,10 +73,12 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=Fal
     L = lib.load()
     dev = torch.device("cuda:0")
     shapes = [(4096, 2048, 1024)] + [(d, d, d) for d in MATMUL_DIMS if d <= max_dim]
+    if dims:   # square sizes of the caller's choice instead of the reference's list
+        shapes = [(d, d, d) for d in dims]
     rows = []
     _settle(dev)
-    # --workspace: the calls lend 4 MiB (kcg_gemm_f32_ws), which sizes with a K-split plan use
-    ws = torch.empty(1 << 20, dtype=torch.float32, device=dev) if workspace else None
+    # --workspace: the calls lend 32 MiB (kcg_gemm_f32_ws), which sizes with a K-split plan use
+    ws = torch.empty(8 << 20, dtype=torch.float32, device=dev) if workspace else None
     for (M, N, K) in shapes:
         if seeded:
             A = torch.from_numpy(inputs.uniform((M, K), MATMUL_SEED, 0)).to(dev)

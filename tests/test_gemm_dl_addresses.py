@@ -100,13 +100,16 @@ def test_streaming_kernel_items_and_addresses(stream_model, case):
 # ---- the launch with K-split tail tiles (kcg_gemm_f32_ws) ----
 @pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048),
                                    (1536, 1536, 4096), (512, 512, 4096), (256, 256, 8192), (512, 1024, 2048),
-                                   (768, 768, 3072), (1280, 1280, 4096), (1344, 1344, 4096)])
+                                   (768, 768, 3072), (1280, 1280, 4096), (1344, 1344, 4096), (640, 640, 1280),
+                                   (1792, 1792, 1792), (2304, 2304, 1152), (3584, 3584, 1024)])
 def test_k_split_launch_numbering_and_addresses(model, shape):
     """The plan kcg_gemm_f32_ws_bytes reports (whole tiles of the full rounds, the rest in
     pieces) replayed on the host: every whole tile and every piece is taken once, a piece
     loads only its own K range, the pieces fill the workspace exactly, and whole tiles plus
-    reduced tiles write every element of C exactly once.  The last four shapes have more
-    pieces than the chip has CUs (672, 432, 1152, 740)."""
+    reduced tiles write every element of C exactly once.  (1280, 1088, 2048), (768, 768, 3072)
+    and the two after it have more pieces than the chip has CUs (672, 432, 1152, 740); the
+    last three are sizes whose plan without a workspace uses a larger tile (3, 5 and 12 full
+    rounds of 64 x 64 tiles before the pieces)."""
     from kernelcodegen_amd import lib
     M, N, K = shape
     need = int(lib.load().kcg_gemm_f32_ws_bytes(M, N, K, None))

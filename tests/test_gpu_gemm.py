@@ -273,13 +273,14 @@ def test_operands_beyond_two_to_the_31_elements(dev):
 @pytest.mark.parametrize("relu", [False, True])
 @pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048),
                                    (512, 512, 4096), (256, 256, 8192), (512, 1024, 2048), (768, 768, 3072),
-                                   (1280, 1280, 4096)])
+                                   (1280, 1280, 4096), (640, 640, 1280), (1792, 1792, 1792)])
 def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
     """Tile counts of whole rounds of the CUs plus a small rest (576 = 2 x 256 + 64; 272 =
     256 + 16; 340 = 256 + 84), and problems with a long K and fewer tiles than CUs (64, 16,
     128, 144 tiles: every tile is cut; 400 = 256 + 144 in eight pieces each: more pieces than
-    CUs): with a workspace the rest is cut along K (2 to 8 pieces) and a second launch adds
-    the pieces up.  Checked against the oracle, against the same
+    CUs; 100 tiles in five pieces; 784 = 3 x 256 + 16, where the plan without a workspace
+    uses 128 x 64 tiles): with a workspace the rest is cut along K (2 to 8 pieces) and a
+    second launch adds the pieces up.  Checked against the oracle, against the same
     call without the workspace (same products, another order of summation), for equal
     results on a second run, and for a workspace that stays inside its bytes."""
     import torch
@@ -318,7 +319,7 @@ def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
 def test_no_k_split_plan_where_it_does_not_pay(dev):
     from kernelcodegen_amd import ops, lib
     for shape in [(4096, 4096, 4096), (1024, 1024, 1024), (512, 512, 512), (1536, 1536, 1500), (1530, 1536, 1536),
-                  (3072, 3072, 3072), (1536, 1536, 256), (1280, 1088, 512)]:
+                  (3072, 3072, 3072), (1536, 1536, 256), (1280, 1088, 512), (512, 512, 768), (576, 576, 576)]:
         assert ops.matmul_workspace_bytes(*shape) == 0, shape
     # a fixed tile keeps its single launch
     assert ops.matmul_workspace_bytes(1536, 1536, 1536, sched=dict(block_m=64, block_n=64, block_k=32, wave_m=32, wave_n=32)) == 0
