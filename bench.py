@@ -13,7 +13,7 @@ launches of the same call) in addition to the --warmup launches, so that the fig
 depend on how many warm-up steps the caller asks for.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
-    python bench.py --sweep matmul [--max-dim D | --dims D1,D2,...] [--relu] [--seeded] [--dump DIR] [--workspace]
+    python bench.py --sweep matmul [--max-dim D | --dims D1,MxNxK,...] [--relu] [--seeded] [--dump DIR] [--workspace]
     python bench.py --sweep fmha | --sweep ops [--shape B,H,S,D]
 """
 import argparse
@@ -127,7 +127,7 @@ def main():
     ap.add_argument("--seeded", action="store_true", help="--sweep matmul: operands from the seeded generator")
     ap.add_argument("--dump", help="--sweep matmul: directory that receives sampled rows of every C")
     ap.add_argument("--dims", default="",
-                    help="--sweep matmul: comma-separated square sizes instead of the reference's list")
+                    help="--sweep matmul: comma-separated sizes instead of the reference's list, each n (square) or MxNxK")
     ap.add_argument("--workspace", action="store_true",
                     help="--sweep matmul: lend the calls a 32 MiB workspace (kcg_gemm_f32_ws)")
     ap.add_argument("--shape", default="1,32,2048,128", help="--sweep ops: B,H,S,D")
@@ -151,7 +151,8 @@ def main():
         from kernelcodegen_amd import sweeps
         if args.sweep == "matmul":
             sweeps.matmul(args.max_dim, args.relu, args.seeded, args.dump, args.workspace,
-                          [int(d) for d in args.dims.split(",")] if args.dims else None)
+                          [int(d) if d.isdigit() else tuple(int(x) for x in d.split("x"))
+                           for d in args.dims.split(",")] if args.dims else None)
         elif args.sweep == "fmha":
             sweeps.fmha()
         else:

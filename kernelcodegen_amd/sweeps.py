@@ -73,8 +73,8 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=Fal
     L = lib.load()
     dev = torch.device("cuda:0")
     shapes = [(4096, 2048, 1024)] + [(d, d, d) for d in MATMUL_DIMS if d <= max_dim]
-    if dims:   # square sizes of the caller's choice instead of the reference's list
-        shapes = [(d, d, d) for d in dims]
+    if dims:   # sizes of the caller's choice instead of the reference's list: n (square) or (M, N, K)
+        shapes = [(d, d, d) if isinstance(d, int) else tuple(d) for d in dims]
     rows = []
     _settle(dev)
     # --workspace: the calls lend 32 MiB (kcg_gemm_f32_ws), which sizes with a K-split plan use
