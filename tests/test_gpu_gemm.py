@@ -316,6 +316,26 @@ def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
         assert not torch.equal(C3, plain)
 
 
+def test_k_split_plan_with_a_group_size(oracle, dev):
+    """GROUP_SIZE_M of the caller's schedule applies to the whole tiles, the pieces and the
+    launch that adds them up alike; the other schedule fields must be left to the library."""
+    import torch
+    from kernelcodegen_amd import ops
+    M, N, K = 1280, 1088, 2048
+    A = inputs.normal((M, K), 433, 0)
+    B = inputs.normal((K, N), 433, 1)
+    ref = oracle.relu(oracle.matmul(A, B))
+    tA, tB = _gpu(A, dev), _gpu(B, dev)
+    ws = torch.empty(ops.matmul_workspace_bytes(M, N, K) // 4, device=dev)
+    base = ops.matmul(tA, tB, relu=True, workspace=ws)
+    for group_m in (1, 3, 4, 16):
+        assert ops.matmul_workspace_bytes(M, N, K, sched=dict(group_m=group_m)) == ws.numel() * 4
+        C = ops.matmul(tA, tB, relu=True, workspace=ws, sched=dict(group_m=group_m))
+        assert max(rel_err(C.cpu().numpy(), ref)) < 1e-4
+        # (other tiles are the remaining ones under another grouping: equal up to summation order)
+        assert max(rel_err(C.cpu().numpy(), base.cpu().numpy())) < 5e-5
+
+
 def test_no_k_split_plan_where_it_does_not_pay(dev):
     from kernelcodegen_amd import ops, lib
     for shape in [(4096, 4096, 4096), (1024, 1024, 1024), (512, 512, 512), (1536, 1536, 1500), (1530, 1536, 1536),
