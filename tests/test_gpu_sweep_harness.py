@@ -56,3 +56,23 @@ def test_output_log_fields_and_rows_against_the_oracle(oracle, dev, tmp_path, re
         assert max(rel_err(got, ref)) < 1e-4, (M, N, K)
     # the summary table carries one row per size
     assert res.stdout.count("\n| %dx%dx%d |" % want[0]) == 1 and res.stdout.count("\n| 1024x1024x1024 |") == 1
+
+
+def test_chosen_sizes_with_a_workspace_against_the_oracle(oracle, dev, tmp_path):
+    """`--dims` (a square size and an M x N x K one) with `--workspace`: 1152^3 runs its
+    K-split plan (the log says so), 512 x 384 x 256 has none; sampled rows of both against
+    the oracle on the same seeded operands."""
+    cmd = [sys.executable, os.path.join(ROOT, "bench.py"), "--sweep", "matmul", "--dims", "1152,512x384x256",
+           "--workspace", "--relu", "--seeded", "--dump", str(tmp_path)]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
+    blocks = BLOCK.findall(res.stdout)
+    want = [(1152, 1152, 1152), (512, 384, 256)]
+    assert [(int(b[0]), int(b[1]), int(b[2])) for b in blocks] == want
+    assert res.stdout.count("K-split plan") == 1
+    for (M, N, K) in want:
+        A = inputs.uniform((M, K), sweeps.MATMUL_SEED, 0)
+        B = inputs.uniform((K, N), sweeps.MATMUL_SEED, 1)
+        got = np.load(os.path.join(str(tmp_path), "C_%dx%dx%d.npy" % (M, N, K)))
+        ref = np.concatenate([oracle.relu(oracle.matmul(np.ascontiguousarray(A[a:c]), B)) for a, c in sweeps.row_bands(M)])
+        assert max(rel_err(got, ref)) < 1e-4, (M, N, K)
