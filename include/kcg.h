@@ -126,8 +126,8 @@ KCG_API int kcg_gemm_f32_query(int64_t M, int64_t N, int64_t K,
 
 /* kcg_gemm_f32 with a workspace lent by the caller.  The reference's generated kernel
  * takes A, B, C only (src/Backend/CUDA.cc:793-801) and every plan of kcg_gemm_f32 keeps to
- * that; one more plan needs device memory for partial sums: where the problem consists of
- * whole 64 x 64 tiles (at most 6400 of them), the tile is left to the library, K is long
+ * that; one more plan needs device memory for partial sums: where K is a multiple of 32 and
+ * N of 4 (any M; at most 6400 tiles of 64 x 64), the tile is left to the library, K is long
  * enough to pay for a second launch and the tile count is some rounds of the compute units
  * plus a rest (1536^3: 2 x 256 + 64; 1792^3: 3 x 256 + 16), or smaller than the number of
  * compute units altogether (512 x 512 x 4096), the tiles of the rest are cut along K into 2

@@ -318,7 +318,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 // per tile.
 // blockIdx.y is the batch index of BatchedMatmul (src/Frontend/Operators.cc:253-420); the
 // three strides are 0 for the plain matmul.
-// SPLIT (full tiles only): the launch holds split_full whole tiles followed by the remaining
+// SPLIT (K in whole slices): the launch holds split_full whole tiles followed by the remaining
 // tiles cut along K into split_parts pieces, one workgroup per piece.  A piece accumulates its
 // K / split_parts slices and writes the raw 64-byte-aligned BM x BN partial tile to
 // ws[(tile - split_full) * split_parts + piece] (no epilogue); gemm_split_reduce_kernel adds
@@ -329,7 +329,7 @@ __device__ __forceinline__ void gemm_dl_body(
     int K, int tiles_m, int tiles_n, int group_m, int64_t batch_a, int64_t batch_b, int64_t batch_c,
     int split_full, int split_parts, float *__restrict__ ws) {
   using T = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N, TRANS_B>;
-  static_assert(!(SPLIT && (RAGGED || TRANS_B)), "K-split pieces exist for full row-major tiles only");
+  static_assert(!(SPLIT && TRANS_B), "K-split pieces exist for row-major B only");
   extern __shared__ __align__(16) float lds[];
   A += blockIdx.y * batch_a;
   B += blockIdx.y * batch_b;
@@ -516,7 +516,9 @@ __device__ __forceinline__ void gemm_dl_body(
   };
 
   const int kfull = my_slices;                   // slices the direct loads may fetch
-  const int ktiles = RAGGED ? (K + BK - 1) / BK : kfull;
+  // (SPLIT: K is a whole number of slices, the host sees to that; RAGGED then means edges
+  // in M and N only)
+  const int ktiles = (RAGGED && !SPLIT) ? (K + BK - 1) / BK : kfull;
   // The last, partial slice (RAGGED): rewritten through registers with zeros beyond K.
   // Lane L of load l owns the same 16 bytes of the stage as in the direct load.
   auto rewrite_tail = [&](int stage_off) {
@@ -680,7 +682,7 @@ __device__ __forceinline__ void gemm_dl_body(
           const int row = m0 + wm * T::kWaveM + 4 * half + local_row;
           float v = acc[i][n][e];
           if (RELU && !to_ws) v = relu_maxf(v);
-          if (!RAGGED || (row < M && col < N)) {
+          if (!RAGGED || to_ws || (row < M && col < N)) {   // a partial tile is stored whole
             float *p = reinterpret_cast<float *>(c_tile + (lane_off + static_cast<unsigned>(local_row) * row_bytes +
                                                            static_cast<unsigned>(n * 32 * 4)));
             if (decltype(stream_c)::value) __builtin_nontemporal_store(v, p);
@@ -704,12 +706,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 }
 
 // The launch with K-split tail tiles (see gemm_dl_body).
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, int MIN_WAVES>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool RAGGED, int MIN_WAVES>
 __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_dl_split_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
     int K, int tiles_m, int tiles_n, int group_m, int split_full, int split_parts, float *__restrict__ ws) {
-  gemm_dl_body<BM, BN, BK, WAVES_M, WAVES_N, RELU, false, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, group_m, 0, 0,
-                                                                       0, split_full, split_parts, ws);
+  gemm_dl_body<BM, BN, BK, WAVES_M, WAVES_N, RELU, RAGGED, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, group_m, 0, 0,
+                                                                        0, split_full, split_parts, ws);
 }
 
 // C tile = epilogue(sum of the split_parts partial tiles).  A tile is shared by
@@ -721,7 +723,7 @@ template <int BM, int BN>
 constexpr int kSplitReduceSlabs = BM * BN / 4 / 256;
 template <int BM, int BN, bool RELU>
 __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *__restrict__ ws, float *__restrict__ C,
-                                                                int N, int tiles_m, int tiles_n, int group_m,
+                                                                int M, int N, int tiles_m, int tiles_n, int group_m,
                                                                 int split_full, int split_parts) {
   constexpr int kSlabs = kSplitReduceSlabs<BM, BN>;
   static_assert(kSlabs * 256 * 4 == BM * BN, "one float4 per thread");
@@ -751,8 +753,9 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *__r
 #pragma unroll
     for (int j = 0; j < 4; ++j) sum[j] = relu_maxf(sum[j]);
   }
-  const int row = idx / (BN / 4), c4 = idx % (BN / 4);
-  *reinterpret_cast<float4_t *>(C + static_cast<int64_t>(m0 + row) * N + n0 + c4 * 4) = sum;
+  // (N is a multiple of 4: a float4 lies inside the matrix or outside it)
+  const int row = m0 + idx / (BN / 4), col = n0 + (idx % (BN / 4)) * 4;
+  if (row < M && col < N) *reinterpret_cast<float4_t *>(C + static_cast<int64_t>(row) * N + col) = sum;
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MIN_WAVES>
@@ -1000,9 +1003,9 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
 }
 
 // ---- K-split tail (the one plan that needs device memory beyond the operands) ----
-// A problem of whole 64 x 64 tiles whose tile count is a few rounds of the CUs plus a small
-// rest (1536^3: 576 = 2 x 256 + 64) holds every CU for one more round on behalf of a quarter
-// of them.  With a workspace the rest is cut along K instead: the launch holds the whole
+// A problem whose 64 x 64 tiles (K in whole slices of 32, N a multiple of 4; edge tiles in M
+// and N allowed) come to a few rounds of the CUs plus a small rest (1536^3: 576 = 2 x 256 +
+// 64) holds every CU for one more round on behalf of a quarter of them.  With a workspace the rest is cut along K instead: the launch holds the whole
 // tiles of the full rounds plus `parts` pieces of each remaining tile, so that every CU gets
 // the same share; the pieces go to the workspace as raw partial tiles and a second, small
 // launch adds them up and applies the epilogue.  The sums are taken in a fixed order: the
@@ -1020,10 +1023,10 @@ struct SplitPlan {
 constexpr int64_t kSplitPieceBytes = 64 * 64 * 4;
 constexpr int64_t kSplitMaxPieces = 2048;   // 32 MiB of partial sums at most
 static bool split_tail_plan(int64_t M, int64_t N, int64_t K, int64_t max_bytes, SplitPlan *out) {
-  if (M % 64 || N % 64 || K % 32 || N >= (1 << 22) || K >= (1 << 22)) return false;
+  if (N % 4 || K % 32 || N >= (1 << 22) || K >= (1 << 22)) return false;
   const TileCand &small = kTileCands[3];
   static_assert(kTileCands[3].bm == 64 && kTileCands[3].bn == 64 && kTileCands[3].bk == 32, "the tile of the split kernel");
-  const int64_t tiles = (M / 64) * (N / 64);
+  const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
   if (static_cast<double>(tiles) > small.max_tiles) return false;
   const int64_t rounds = tiles / kNumCu, rest = tiles % kNumCu;
   if (rest == 0) return false;
@@ -1063,23 +1066,26 @@ static bool split_tail_plan(int64_t M, int64_t N, int64_t K, int64_t max_bytes, 
 static int launch_split(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
                         int group_m, const SplitPlan &sp, float *ws, hipStream_t stream) {
   using TD = GemmDlTile<64, 64, 32, 2, 2>;
-  const int tiles_m = static_cast<int>(M / 64), tiles_n = static_cast<int>(N / 64);
+  const int tiles_m = static_cast<int>((M + 63) / 64), tiles_n = static_cast<int>((N + 63) / 64);
   const bool relu = epilogue == KCG_EPILOGUE_RELU;
+  const bool ragged = M % 64 != 0 || N % 64 != 0;
   const dim3 grid(static_cast<unsigned>(sp.full + sp.rest * sp.parts)), block(256);
   auto main_launch = [&](auto kern) {
     if (!allow_lds(kern, TD::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
     return launch(kern, grid, block, TD::kLdsBytes, stream, A, B, C, static_cast<int>(M), static_cast<int>(N),
                   static_cast<int>(K), tiles_m, tiles_n, group_m, sp.full, sp.parts, ws);
   };
-  const int st = relu ? main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, true, 2>)
-                      : main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, false, 2>);
+  const int st = ragged ? (relu ? main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, true, true, 2>)
+                                : main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, false, true, 2>))
+                        : (relu ? main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, true, false, 2>)
+                                : main_launch(gemm_f32_dl_split_kernel<64, 64, 32, 2, 2, false, false, 2>));
   if (st != KCG_OK) return st;
   const float *cws = ws;
   const dim3 reduce_grid(static_cast<unsigned>(sp.rest * kSplitReduceSlabs<64, 64>));
   return relu ? launch(gemm_split_reduce_kernel<64, 64, true>, reduce_grid, dim3(256), 0, stream, cws, C,
-                       static_cast<int>(N), tiles_m, tiles_n, group_m, sp.full, sp.parts)
+                       static_cast<int>(M), static_cast<int>(N), tiles_m, tiles_n, group_m, sp.full, sp.parts)
               : launch(gemm_split_reduce_kernel<64, 64, false>, reduce_grid, dim3(256), 0, stream, cws, C,
-                       static_cast<int>(N), tiles_m, tiles_n, group_m, sp.full, sp.parts);
+                       static_cast<int>(M), static_cast<int>(N), tiles_m, tiles_n, group_m, sp.full, sp.parts);
 }
 
 // The schedule leaves the tile to the library (only GROUP_SIZE_M may be set).

@@ -224,14 +224,16 @@ int replay(int64_t M64, int64_t N64, int64_t K64, int group_m) {
 // gemm_split_reduce_kernel): `full` whole tiles, then every remaining tile in `parts` pieces.
 // Checks the two-set numbering (every whole tile and every (tile, piece) exactly once), the K
 // range every piece loads, that the pieces fill the workspace exactly, and that whole tiles
-// plus reduced tiles write every element of C exactly once.
+// plus reduced tiles write every element of C exactly once.  M and N need not be multiples of
+// the tile (edge tiles clamp their loads and bound their stores to C; partial tiles go to
+// the workspace whole); K is a whole number of slices and N a multiple of 4.
 int replay_split(int64_t M64, int64_t N64, int64_t K64, int group_m, int full, int parts) {
   constexpr int BM = 64, BN = 64, BK = 32, WAVES_N = 2;
   using T = kcg::GemmDlTile<BM, BN, BK, 2, 2, false>;
   const int M = static_cast<int>(M64), N = static_cast<int>(N64), K = static_cast<int>(K64);
-  if (M % BM || N % BN || K % BK) return 2;
+  if (N % 4 || K % BK) return 2;
   const int64_t bytes_a = M64 * K64 * 4, bytes_b = K64 * N64 * 4;
-  const int tiles_m = M / BM, tiles_n = N / BN, tiles = tiles_m * tiles_n;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN, tiles = tiles_m * tiles_n;
   const int rest = tiles - full;
   if (full % 8 || rest <= 0 || parts < 2 || (K / BK) % parts) return 2;
   const int grid = full + rest * parts;
@@ -263,7 +265,7 @@ int replay_split(int64_t M64, int64_t N64, int64_t K64, int group_m, int full, i
     }
     int m0, n0;
     origin(logical, &m0, &n0);
-    if (m0 < 0 || m0 + BM > M || n0 < 0 || n0 + BN > N) fail("tile origin", wg, 0, 0, m0);
+    if (m0 < 0 || m0 >= M || n0 < 0 || n0 >= N) fail("tile origin", wg, 0, 0, m0);
     const int my_slices = partial ? (K / BK) / parts : K / BK;
     const int64_t b_step = static_cast<int64_t>(BK) * N * 4;
     const int64_t ga0 = static_cast<int64_t>(m0) * K * 4 + static_cast<int64_t>(piece) * my_slices * (BK * 4);
@@ -279,7 +281,8 @@ int replay_split(int64_t M64, int64_t N64, int64_t K64, int group_m, int full, i
         for (int i = 0; i < T::kInstrA; ++i) {
           const int idx = (wave * T::kInstrA + i) * 256 + lane * 4;
           const int row = idx / BK;
-          const unsigned oa = as_u32((static_cast<int64_t>(row) * K + 4 * (((idx % BK) / 4) ^ T::fa(row))) * 4, "oa", wg, wave, lane);
+          const int grow = row < M - m0 ? row : M - m0 - 1;   // rows at and beyond M fetch the last valid row
+          const unsigned oa = as_u32((static_cast<int64_t>(grow) * K + 4 * (((idx % BK) / 4) ^ T::fa(row))) * 4, "oa", wg, wave, lane);
           for (int64_t basep : {ga0, ga1}) {
             const int64_t addr = basep + oa;
             if (addr < 0 || addr + 16 > bytes_a) fail("A load out of range", wg, wave, lane, addr);
@@ -289,7 +292,9 @@ int replay_split(int64_t M64, int64_t N64, int64_t K64, int group_m, int full, i
         }
         for (int i = 0; i < T::kInstrB; ++i) {
           const int idx = (wave * T::kInstrB + i) * 256 + lane * 4;
-          const unsigned ob = as_u32((static_cast<int64_t>(idx / BN) * N + idx % BN) * 4, "ob", wg, wave, lane);
+          const int col = idx % BN;
+          const int gcol = col < N - n0 ? col : N - n0 - 4;   // column chunks at and beyond N fetch the last valid chunk
+          const unsigned ob = as_u32((static_cast<int64_t>(idx / BN) * N + gcol) * 4, "ob", wg, wave, lane);
           for (int64_t basep : {gb0, gb1}) {
             const int64_t addr = basep + ob;
             if (addr < 0 || addr + 16 > bytes_b) fail("B load out of range", wg, wave, lane, addr);
@@ -313,7 +318,11 @@ int replay_split(int64_t M64, int64_t N64, int64_t K64, int group_m, int full, i
                 const int row = wm * T::kWaveM + 4 * half + local_row, col = wn * T::kWaveN + n * 32 + r32;
                 if (static_cast<int64_t>(off32 / 4) != static_cast<int64_t>(row) * BN + col) fail("partial tile layout", wg, wave, lane, off32);
               } else {
+                // whole tiles at the edges of C store only what lies inside it
+                const int grow = m0 + wm * T::kWaveM + 4 * half + local_row, gcol = n0 + wn * T::kWaveN + n * 32 + r32;
+                if (grow >= M || gcol >= N) continue;
                 const int64_t el = (static_cast<int64_t>(m0) * N + n0) + off32 / 4;
+                if (el != static_cast<int64_t>(grow) * N + gcol) fail("C store target", wg, wave, lane, el);
                 if (el < 0 || el >= static_cast<int64_t>(M) * N) fail("C store out of range", wg, wave, lane, el);
                 else if (c_written[static_cast<size_t>(el)]++) fail("C element written twice", wg, wave, lane, el);
               }
@@ -334,10 +343,11 @@ int replay_split(int64_t M64, int64_t N64, int64_t K64, int group_m, int full, i
         const int64_t fl = static_cast<int64_t>(j) * parts * (BM * BN) + idx * 4 + static_cast<int64_t>(p < parts ? p : 0) * (BM * BN);
         if (fl < 0 || fl + 4 > ws_floats) fail("reduce read out of range", j, 0, 0, fl);
       }
-      const int row = idx / (BN / 4), c4 = idx % (BN / 4);
+      const int row = m0 + idx / (BN / 4), col = n0 + (idx % (BN / 4)) * 4;
+      if (row >= M || col >= N) continue;   // the float4 lies outside C (N is a multiple of 4)
       for (int x = 0; x < 4; ++x) {
-        const int64_t el = static_cast<int64_t>(m0 + row) * N + n0 + c4 * 4 + x;
-        if (el < 0 || el >= static_cast<int64_t>(M) * N) fail("reduce store out of range", j, 0, 0, el);
+        const int64_t el = static_cast<int64_t>(row) * N + col + x;
+        if (col + x >= N || el < 0 || el >= static_cast<int64_t>(M) * N) fail("reduce store out of range", j, 0, 0, el);
         else if (c_written[static_cast<size_t>(el)]++) fail("C element written twice (reduce)", j, 0, 0, el);
       }
     }

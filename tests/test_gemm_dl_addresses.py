@@ -101,7 +101,8 @@ def test_streaming_kernel_items_and_addresses(stream_model, case):
 @pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048),
                                    (1536, 1536, 4096), (512, 512, 4096), (256, 256, 8192), (512, 1024, 2048),
                                    (768, 768, 3072), (1280, 1280, 4096), (1344, 1344, 4096), (640, 640, 1280),
-                                   (1792, 1792, 1792), (2304, 2304, 1152), (3584, 3584, 1024)])
+                                   (1792, 1792, 1792), (2304, 2304, 1152), (3584, 3584, 1024),
+                                   (1500, 1500, 1536), (300, 260, 4096), (1000, 1500, 2048), (1530, 1536, 1536)])
 def test_k_split_launch_numbering_and_addresses(model, shape):
     """The plan kcg_gemm_f32_ws_bytes reports (whole tiles of the full rounds, the rest in
     pieces) replayed on the host: every whole tile and every piece is taken once, a piece
@@ -109,11 +110,11 @@ def test_k_split_launch_numbering_and_addresses(model, shape):
     reduced tiles write every element of C exactly once.  (1280, 1088, 2048), (768, 768, 3072)
     and the two after it have more pieces than the chip has CUs (672, 432, 1152, 740); the
     last three are sizes whose plan without a workspace uses a larger tile (3, 5 and 12 full
-    rounds of 64 x 64 tiles before the pieces)."""
+    rounds of 64 x 64 tiles before the pieces); the last four have edge tiles in M, N or both."""
     from kernelcodegen_amd import lib
     M, N, K = shape
     need = int(lib.load().kcg_gemm_f32_ws_bytes(M, N, K, None))
-    tiles = (M // 64) * (N // 64)
+    tiles = ((M + 63) // 64) * ((N + 63) // 64)
     rest = tiles % 256
     assert need > 0 and need % (rest * 64 * 64 * 4) == 0
     parts = need // (rest * 64 * 64 * 4)

@@ -273,13 +273,15 @@ def test_operands_beyond_two_to_the_31_elements(dev):
 @pytest.mark.parametrize("relu", [False, True])
 @pytest.mark.parametrize("shape", [(1536, 1536, 1536), (1536, 1536, 1024), (1024, 1088, 1536), (1280, 1088, 2048),
                                    (512, 512, 4096), (256, 256, 8192), (512, 1024, 2048), (768, 768, 3072),
-                                   (1280, 1280, 4096), (640, 640, 1280), (1792, 1792, 1792)])
+                                   (1280, 1280, 4096), (640, 640, 1280), (1792, 1792, 1792), (1500, 1500, 1536),
+                                   (300, 260, 4096), (1000, 1500, 2048)])
 def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
     """Tile counts of whole rounds of the CUs plus a small rest (576 = 2 x 256 + 64; 272 =
     256 + 16; 340 = 256 + 84), and problems with a long K and fewer tiles than CUs (64, 16,
     128, 144 tiles: every tile is cut; 400 = 256 + 144 in eight pieces each: more pieces than
     CUs; 100 tiles in five pieces; 784 = 3 x 256 + 16, where the plan without a workspace
-    uses 128 x 64 tiles): with a workspace the rest is cut along K (2 to 8 pieces) and a
+    uses 128 x 64 tiles; the last three have edge tiles: M and N need not be multiples of 64,
+    only N of 4 and K of 32): with a workspace the rest is cut along K (2 to 8 pieces) and a
     second launch adds the pieces up.  Checked against the oracle, against the same
     call without the workspace (same products, another order of summation), for equal
     results on a second run, and for a workspace that stays inside its bytes."""
@@ -303,7 +305,7 @@ def test_k_split_plan_with_a_workspace(oracle, dev, shape, relu):
     plain = ops.matmul(tA, tB, relu=relu)
     assert max(rel_err(C1.cpu().numpy(), plain.cpu().numpy())) < 5e-5
     # a workspace too small for any plan is not used: the call is the plain one, bit for bit
-    assert need // 8 < (M // 64) * (N // 64) % 256 * 2 * 64 * 64 * 4   # not even two pieces per tile
+    assert need // 8 < ((M + 63) // 64) * ((N + 63) // 64) % 256 * 2 * 64 * 64 * 4   # not even two pieces per tile
     small = ops.matmul(tA, tB, relu=relu, workspace=buf[:need // 8 // 4])
     assert torch.equal(small, plain)
     if shape == (1280, 1088, 2048):
@@ -338,7 +340,7 @@ def test_k_split_plan_with_a_group_size(oracle, dev):
 
 def test_no_k_split_plan_where_it_does_not_pay(dev):
     from kernelcodegen_amd import ops, lib
-    for shape in [(4096, 4096, 4096), (1024, 1024, 1024), (512, 512, 512), (1536, 1536, 1500), (1530, 1536, 1536),
+    for shape in [(4096, 4096, 4096), (1024, 1024, 1024), (512, 512, 512), (1536, 1536, 1500), (1536, 1530, 1536),
                   (3072, 3072, 3072), (1536, 1536, 256), (1280, 1088, 512), (512, 512, 768), (576, 576, 576)]:
         assert ops.matmul_workspace_bytes(*shape) == 0, shape
     # a fixed tile keeps its single launch
