@@ -146,6 +146,16 @@ KCG_API int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M,
                             const kcg_gemm_sched *sched, void *workspace,
                             int64_t workspace_bytes, void *stream);
 
+/* Launch geometry of kcg_gemm_f32_ws for a workspace of `workspace_bytes` (the counterpart
+ * of kcg_gemm_f32_query, same logging purpose, src/Backend/CUDA.cc:786-791).  Where the
+ * K-split plan runs, launches == 2: grid / block / lds_bytes / kernel describe the launch
+ * of whole tiles and pieces (main_rows = M, tail_rows = 0: both launches cover all rows),
+ * the tail_* fields the launch that adds the pieces up.  Otherwise the answer is that of
+ * kcg_gemm_f32_query.  For kcg_gemm_f32_noalloc pass 4 MiB. */
+KCG_API int kcg_gemm_f32_ws_query(int64_t M, int64_t N, int64_t K,
+                                  const kcg_gemm_sched *sched, int64_t workspace_bytes,
+                                  kcg_launch_info *out);
+
 /* kcg_gemm_f32_ws without a workspace argument and without any allocation.  It has no
  * counterpart in the reference; it is for callers that can neither allocate device memory
  * nor lend any: code under HIP graph capture, tight serving loops, harnesses that forbid
@@ -155,7 +165,12 @@ KCG_API int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M,
  * more pieces are not considered, a plan that did not fit would be refused with
  * KCG_ERR_UNSUPPORTED_SHAPE).  All calls on one GPU share that array: calls that overlap in
  * time on one GPU (two streams, two threads) race on it and must be serialised by the
- * caller.  Same arguments, statuses and results as kcg_gemm_f32_ws with 4 MiB. */
+ * caller.  Same arguments, statuses and results as kcg_gemm_f32_ws with 4 MiB.
+ * The first call on a device looks up the array's address (hipGetSymbolAddress), and the
+ * first launch of a kernel variant that needs more than 48 KiB of LDS raises that kernel's
+ * limit (hipFuncSetAttribute): make one call per device and problem class outside graph
+ * capture before capturing one; under capture the call then only launches kernels (no
+ * memset node is recorded). */
 KCG_API int kcg_gemm_f32_noalloc(const float *A, const float *B, float *C, int64_t M,
                                  int64_t N, int64_t K, int epilogue,
                                  const kcg_gemm_sched *sched, void *stream);
@@ -189,7 +204,16 @@ typedef enum kcg_dtype { KCG_F32 = 0, KCG_BF16 = 1 } kcg_dtype;
 /* Same, with Q, K, V holding bf16 bit patterns (extension: the reference knows
  * only float32/float64/float16, src/Frontend/Operators.cc:5-10).  Products are
  * bf16 x bf16 accumulated in fp32; softmax in fp32; P is rounded to bf16 before
- * the second product.  O is written as o_dtype (KCG_BF16 or KCG_F32). */
+ * the second product.  O is written as o_dtype (KCG_BF16 or KCG_F32).
+ *
+ * Deviation from the fp32 evaluation of the same bf16 inputs: the weights of a row
+ * are rounded to bf16 (unit roundoff 2^-8) and the row is normalised by the sum of
+ * the rounded weights, so every element obeys
+ *   |O - O_fp32| <= 2^-8 (sum_j P_ij |V_jd| + |O_id|)   (P the normalised weights)
+ * up to fp32 rounding, plus 2^-8 |O_id| when O is written as bf16.  For rows that
+ * average many keys this is far inside 2e-2 of the output's RMS; a causal row that
+ * sees only a handful of keys with cancelling V values can reach 2.4e-2 of that RMS
+ * on single elements (it stays inside the bound above and inside 2e-2 of max|O|). */
 KCG_API int kcg_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                           void *O, int o_dtype, int32_t B, int32_t H, int32_t S,
                           int32_t D, float scale, int causal,

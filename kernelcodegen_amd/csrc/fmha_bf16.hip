@@ -109,7 +109,7 @@ constexpr float kTau = 8.0f;
 // POS_SCALE: scale > 0, so exp2(s * c - m) is one FMA and the row maximum can be
 // taken on the raw products.  The general variant scales first.
 template <int D, int BC, int QT, int WAVES, bool CAUSAL, bool OUT_BF16, bool POS_SCALE>
-__global__ __launch_bounds__(64 * WAVES, (QT == 1 ? 2 : 1)) void fmha_bf16_kernel(
+__global__ __launch_bounds__(64 * WAVES, (QT == 1 && WAVES > 2 ? 2 : 1)) void fmha_bf16_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     void *__restrict__ O, int S, int q_blocks, int q_items, float scale_log2e) {
   using T = FmhaBf16Tile<D, BC, QT, WAVES>;
@@ -291,7 +291,12 @@ __global__ __launch_bounds__(64 * WAVES, (QT == 1 ? 2 : 1)) void fmha_bf16_kerne
 #pragma unroll
           for (int ds = 0; ds < T::kDSteps; ++ds) {
             if (ds + kAhead < T::kDSteps) fetch(ds + kAhead);
-            if (ds < 2 * T::kIpw && spread) load_one(kv_nxt, nxt, ds);
+            // (one direct load per d-step in the 4- and 8-wave tiles; the two-wave 64 x 128
+            // tile has four times as many loads per wave)
+            constexpr int kLoadsPerDs = (2 * T::kIpw + T::kDSteps - 1) / T::kDSteps;
+#pragma unroll
+            for (int j = 0; j < kLoadsPerDs; ++j)
+              if (ds * kLoadsPerDs + j < 2 * T::kIpw && spread) load_one(kv_nxt, nxt, ds * kLoadsPerDs + j);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kt = 0; kt < T::kKeyTiles; ++kt)
@@ -1056,10 +1061,18 @@ int dispatch_fmha_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V, 
     if (sched->br) br = sched->br;
     if (sched->bc) bc = sched->bc;
   }
-  if (bc != 64) return KCG_ERR_BAD_SCHEDULE;
-  if (br != 128 && br != 256) return KCG_ERR_BAD_SCHEDULE;
+  // (Br 64 x Bc 128 is the tile the reference's own table gives at Hd = 128, include/
+  // KernelCodeGen.h:38-41, src/Optimizer/Optimizer.cc:1136-1144: two waves on the 128-row
+  // kernel's code, built so that the reference's literal configuration binds)
+  const bool reference_tile = D == 128 && br == 64 && bc == 128;
+  if (bc != 64 && !reference_tile) return KCG_ERR_BAD_SCHEDULE;
+  if (br != 128 && br != 256 && !reference_tile) return KCG_ERR_BAD_SCHEDULE;
   // scale <= 0 takes the general softmax path, built for the 128-row block only
   const bool pos = scale > 0.0f;
+  if (reference_tile) {
+    if (pos) return launch_fmha_bf16<128, 128, 1, 2, true>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, info);
+    return launch_fmha_bf16<128, 128, 1, 2, false>(Q, K, V, O, o_dtype, B, H, S, scale, causal, stream, info);
+  }
 #define KCG_PICK(D_)                                                                              \
   if (D == D_) {                                                                                  \
     if (!pos)                                                                                     \

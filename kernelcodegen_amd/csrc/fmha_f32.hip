@@ -62,7 +62,7 @@ struct FmhaF32Tile {
 constexpr float kTau = 8.0f;
 
 template <int D, int BC, int WAVES, bool CAUSAL>
-__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fmha_f32_kernel(const float *__restrict__ Q,
+__global__ __launch_bounds__(64 * WAVES, WAVES == 2 ? 1 : 8 / WAVES) void fmha_f32_kernel(const float *__restrict__ Q,
                                                           const float *__restrict__ K,
                                                           const float *__restrict__ V,
                                                           float *__restrict__ O, int S,
@@ -392,14 +392,19 @@ int dispatch_fmha_f32(const float *Q, const float *K, const float *V, float *O, 
     if (sched->br) br = sched->br;
     if (sched->bc) bc = sched->bc;
   }
-  if (br != 128 && br != 256) return KCG_ERR_BAD_SCHEDULE;
-  if (bc != 32 && bc != 64) return KCG_ERR_BAD_SCHEDULE;
+  // (Br 64 x Bc 128 is the tile the reference's own table gives at Hd = 128: Br = 8192 / Hd,
+  // Bc = 8192 / Br, include/KernelCodeGen.h:38-41, src/Optimizer/Optimizer.cc:1136-1144;
+  // at Hd = 64 that table gives 128 x 64)
+  const bool reference_tile = D == 128 && br == 64 && bc == 128;
+  if (br != 128 && br != 256 && !reference_tile) return KCG_ERR_BAD_SCHEDULE;
+  if (bc != 32 && bc != 64 && !reference_tile) return KCG_ERR_BAD_SCHEDULE;
 #define KCG_PICK(D_, BC_, WAVES_)                \
   if (D == D_ && bc == BC_ && br == 32 * WAVES_) \
     return launch_fmha_f32<D_, BC_, WAVES_>(Q, K, V, O, B, H, S, scale, causal, stream, info);
   KCG_PICK(128, 32, 4)
   KCG_PICK(128, 32, 8)
   KCG_PICK(128, 64, 4)
+  KCG_PICK(128, 128, 2)
   KCG_PICK(64, 32, 4)
   KCG_PICK(64, 32, 8)
   KCG_PICK(64, 64, 4)

@@ -1099,6 +1099,10 @@ static bool tile_is_free(const kcg_gemm_sched *s) {
 // and the workspace holds it, the plain plan otherwise.
 static int dispatch_gemm_ws(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
                             const kcg_gemm_sched *s, float *ws, int64_t ws_bytes, hipStream_t stream) {
+  // (the plain path refuses a GROUP_SIZE_M below 1 in launch_sched; the split launch numbers
+  // its tiles with the same value and must refuse it too: a negative one turns the tile
+  // origins negative)
+  if (s && s->group_m < 0) return KCG_ERR_BAD_SCHEDULE;
   SplitPlan sp;
   if (ws && tile_is_free(s) && split_tail_plan(M, N, K, ws_bytes, &sp) && aligned16(A) &&
       aligned16(B) && aligned16(C) && aligned16(ws))
@@ -1260,11 +1264,43 @@ int kcg_gemm_f32_ws(const float *A, const float *B, float *C, int64_t M, int64_t
                                static_cast<hipStream_t>(stream));
 }
 
+int kcg_gemm_f32_ws_query(int64_t M, int64_t N, int64_t K, const kcg_gemm_sched *sched, int64_t workspace_bytes,
+                          kcg_launch_info *out) {
+  if (!out) return KCG_ERR_NULL_POINTER;
+  if (const int st = gemm_shape_status(M, N, K)) return st;
+  if (workspace_bytes < 0) return KCG_ERR_BAD_ARGUMENT;
+  if (sched && sched->group_m < 0) return KCG_ERR_BAD_SCHEDULE;
+  kcg::SplitPlan sp;
+  if (!kcg::tile_is_free(sched) || !kcg::split_tail_plan(M, N, K, workspace_bytes, &sp))
+    return kcg::dispatch_gemm(nullptr, nullptr, nullptr, M, N, K, KCG_EPILOGUE_NONE, sched, nullptr, out);
+  // the two launches of kcg::launch_split: whole tiles and pieces, then the adding launch
+  using TD = kcg::GemmDlTile<64, 64, 32, 2, 2>;
+  *out = kcg_launch_info{};
+  out->launches = 2;
+  out->grid[0] = sp.full + sp.rest * sp.parts;
+  out->grid[1] = out->grid[2] = 1;
+  out->block[0] = 256;
+  out->block[1] = out->block[2] = 1;
+  out->lds_bytes = TD::kLdsBytes;
+  out->waves_per_block = 4;
+  snprintf(out->kernel, sizeof out->kernel, "gemm_f32_dl_split_64x64x32_full%d_rest%dx%d", sp.full, sp.rest, sp.parts);
+  out->main_rows = static_cast<int32_t>(M);
+  out->tail_rows = 0;
+  out->tail_grid[0] = sp.rest * kcg::kSplitReduceSlabs<64, 64>;
+  out->tail_grid[1] = out->tail_grid[2] = 1;
+  out->tail_block[0] = 256;
+  out->tail_block[1] = out->tail_block[2] = 1;
+  out->tail_lds_bytes = 0;
+  snprintf(out->tail_kernel, sizeof out->tail_kernel, "gemm_split_reduce_64x64_parts%d", sp.parts);
+  return KCG_OK;
+}
+
 int kcg_gemm_f32_noalloc(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
                          const kcg_gemm_sched *sched, void *stream) {
   if (!A || !B || !C) return KCG_ERR_NULL_POINTER;
   if (const int st = gemm_shape_status(M, N, K)) return st;
   if (epilogue != KCG_EPILOGUE_NONE && epilogue != KCG_EPILOGUE_RELU) return KCG_ERR_BAD_ARGUMENT;
+  if (sched && sched->group_m < 0) return KCG_ERR_BAD_SCHEDULE;
   // the plan is looked for among those whose partial sums fit the array; where there is none
   // the call is the plain one, which uses no memory of its own
   kcg::SplitPlan sp;

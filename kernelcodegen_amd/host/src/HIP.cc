@@ -2,11 +2,13 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <iostream>
 #include <set>
 #include <sstream>
 
 #include "Optimizer/Analyzer.h"
+#include "Optimizer/Optimizer.h"
 #include "enum.h"
 
 namespace KernelCodeGen {
@@ -182,22 +184,151 @@ bool bindFmha(FuncOp f, KernelBinding &b) {
   return true;
 }
 
+size_t bytesOf(const MemRefType &t) {
+  const size_t elem = t.elem == DType::f64 ? 8 : (t.elem == DType::f32 ? 4 : 2);
+  return static_cast<size_t>(t.numElements()) * elem;
+}
+
+bool allF32(FuncOp f) {
+  for (auto a : f.getArguments())
+    if (!a.isMemRef() || a.getMemRefType().elem != DType::f32) return false;
+  return true;
+}
+
+// Relu_Elementwise_<dims> (src/Frontend/Operators.cc:182-250): one memref in; the result is
+// that memref (MemorySpace::inplace) or a buffer the function allocates itself.
+bool bindRelu(FuncOp f, KernelBinding &b) {
+  auto args = f.getArguments();
+  if (args.size() != 1 || !allF32(f)) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": only the float32 Relu has a gfx950 kernel\n";
+    return false;
+  }
+  b.kind = KernelBinding::Relu;
+  b.entry = "kcg_relu_f32";
+  b.count = args[0].getMemRefType().numElements();
+  // in place when the function returns its own argument
+  b.inPlace = true;
+  walk(f.op, [&](Op *o) {
+    if (o->kind == OpKind::Return && !o->operands.empty() && o->operands[0] != args[0]) b.inPlace = false;
+  });
+  b.argNames = b.inPlace ? std::vector<std::string>{"x"} : std::vector<std::string>{"x", "y"};
+  b.argBytes.assign(b.argNames.size(), bytesOf(args[0].getMemRefType()));
+  return true;
+}
+
+// BatchMatmul_<batch..>_m<M>_n<N>_k<K>_<N|T><N|T> (src/Frontend/Operators.cc:253-420; the
+// name is parsed back as the reference's optimizer does, src/Optimizer/Optimizer.cc:564-584).
+bool bindBatchedMatmul(FuncOp f, KernelBinding &b) {
+  auto args = f.getArguments();
+  BatchMatmulDescriptor d;
+  if (args.size() != 3 || !identifyBatchMatmul(f.getSymName(), d)) return false;
+  if (!allF32(f)) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": only the float32 BatchedMatmul has a gfx950 kernel\n";
+    return false;
+  }
+  b.kind = KernelBinding::BatchedMatmul;
+  b.entry = "kcg_batched_matmul_f32";
+  b.batch = 1;
+  for (int x : d.batch) b.batch *= x;
+  b.M = d.m;
+  b.N = d.n;
+  b.K = d.k;
+  b.transA = d.transA ? 1 : 0;
+  b.transB = d.transB ? 1 : 0;
+  b.argNames = {"A", "B", "C"};
+  for (auto a : args) b.argBytes.push_back(bytesOf(a.getMemRefType()));
+  if (b.argBytes[0] != static_cast<size_t>(b.batch * b.M * b.K) * 4 ||
+      b.argBytes[1] != static_cast<size_t>(b.batch * b.K * b.N) * 4 ||
+      b.argBytes[2] != static_cast<size_t>(b.batch * b.M * b.N) * 4) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": the operand types do not have the extents the name encodes\n";
+    return false;
+  }
+  return true;
+}
+
+// Softmax_<dims>_axis<k> (src/Frontend/Operators.cc:425-542): last axis only, in place.
+bool bindSoftmax(FuncOp f, KernelBinding &b) {
+  auto args = f.getArguments();
+  if (args.size() != 1 || !allF32(f)) {
+    std::cerr << "HIPBind: " << f.getSymName() << ": only the float32 Softmax has a gfx950 kernel\n";
+    return false;
+  }
+  const MemRefType &t = args[0].getMemRefType();
+  const std::string &name = f.getSymName();
+  const size_t at = name.rfind("_axis");
+  if (t.shape.empty() || at == std::string::npos ||
+      std::atoi(name.c_str() + at + 5) != static_cast<int>(t.shape.size()) - 1) {
+    std::cerr << "HIPBind: " << name << ": the kernel reduces over the last axis only\n";
+    return false;
+  }
+  b.kind = KernelBinding::Softmax;
+  b.entry = "kcg_softmax_f32";
+  b.rowLength = t.shape.back();
+  b.count = t.numElements();
+  b.inPlace = true;
+  b.argNames = {"x"};
+  b.argBytes = {bytesOf(t)};
+  return true;
+}
+
 }  // namespace
+
+Value HIPBufferOf(ModuleOp &module, Value v) {
+  for (int hops = 0; hops < 1024 && v; ++hops) {
+    Op *def = v.getDefiningOp();
+    if (!def || def->kind != OpKind::Call) return v;   // an allocation of the module
+    FuncOp f = Analyzer::getTargetFunction(module, def->name);
+    if (!f) return v;
+    // which argument the function returns: Matmul / BatchMatmul return C (their last
+    // argument), Softmax and the in-place Relu their only one, the fused attention O
+    auto args = f.getArguments();
+    int returned = -1;
+    walk(f.op, [&](Op *o) {
+      if (o->kind != OpKind::Return || o->operands.empty()) return;
+      for (size_t i = 0; i < args.size(); ++i)
+        if (o->operands[0] == args[i]) returned = static_cast<int>(i);
+    });
+    if (returned < 0 || returned >= static_cast<int>(def->operands.size())) return v;  // a buffer of its own
+    v = def->operands[returned];
+  }
+  return v;
+}
 
 std::vector<KernelBinding> HIPBind(ModuleOp &module) {
   std::vector<KernelBinding> out;
   // module order of the calls decides kernel numbering, as the emitter numbers kernels in walk order
   for (auto call : Analyzer::collectFuncCalls(module)) {
     FuncOp f = Analyzer::getTargetFunction(module, call.getCallee());
-    if (!f || f.getAttr("func.state") != "gpu") continue;
+    if (!f) continue;
+    const std::string state = f.getAttr("func.state");
     KernelBinding b;
     b.graph = module.getName();
     b.funcName = f.getSymName();
     bool ok = false;
-    if (b.funcName.rfind("Matmul_m", 0) == 0) ok = bindMatmul(f, b);
-    else if (b.funcName.rfind("Fused_Multi_Head_Attention", 0) == 0) ok = bindFmha(f, b);
-    else std::cerr << "HIPBind: no gfx950 kernel is bound to " << b.funcName << "\n";
+    if (state == "gpu") {
+      if (b.funcName.rfind("Matmul_m", 0) == 0) ok = bindMatmul(f, b);
+      else if (b.funcName.rfind("Fused_Multi_Head_Attention", 0) == 0) ok = bindFmha(f, b);
+      else std::cerr << "HIPBind: no gfx950 kernel is bound to " << b.funcName << "\n";
+      if (ok)
+        for (auto a : f.getArguments()) b.argBytes.push_back(bytesOf(a.getMemRefType()));
+    } else if (state == "cpu") {
+      // no pattern matched this call: the un-fused kernels
+      if (b.funcName.rfind("Relu_Elementwise", 0) == 0) ok = bindRelu(f, b);
+      else if (b.funcName.rfind("BatchMatmul_", 0) == 0) ok = bindBatchedMatmul(f, b);
+      else if (b.funcName.rfind("Softmax_", 0) == 0) ok = bindSoftmax(f, b);
+      else std::cerr << "HIPBind: no gfx950 kernel is bound to " << b.funcName << "\n";
+      if (ok) snprintf(b.launch.kernel, sizeof b.launch.kernel, "%s", b.entry.c_str());
+    } else {
+      continue;
+    }
     if (!ok) continue;
+    for (auto v : call.getArgOperands()) b.buffers.push_back(HIPBufferOf(module, v));
+    if (b.kind == KernelBinding::Relu && !b.inPlace) b.buffers.push_back(call.getResult(0));
+    if (b.buffers.size() != b.argNames.size()) {
+      std::cerr << "HIPBind: " << b.funcName << ": the call has " << b.buffers.size() << " operands, the kernel takes "
+                << b.argNames.size() << "\n";
+      continue;
+    }
     b.index = static_cast<int>(out.size());
     out.push_back(b);
   }
@@ -213,6 +344,25 @@ std::string HIPGen(ModuleOp &module) {
      << "#include \"kcg.h\"\n\n"
      << "namespace " << module.getName() << " {\n\n";
   for (auto &b : bindings) {
+    if (b.kind == KernelBinding::Relu || b.kind == KernelBinding::BatchedMatmul || b.kind == KernelBinding::Softmax) {
+      os << "// " << b.funcName << " -> " << b.entry << " (un-fused operator: no pattern matched this call; "
+         << "the library picks the launch geometry from the extents)\n";
+      if (b.kind == KernelBinding::Relu && b.inPlace)
+        os << "inline int kernel" << b.index << "(float* arg0 /*x, in place*/, void* stream = nullptr) {\n"
+           << "  return kcg_relu_f32(arg0, arg0, " << b.count << ", stream);\n}\n\n";
+      else if (b.kind == KernelBinding::Relu)
+        os << "inline int kernel" << b.index << "(const float* arg0 /*x*/, float* arg1 /*y*/, void* stream = nullptr) {\n"
+           << "  return kcg_relu_f32(arg0, arg1, " << b.count << ", stream);\n}\n\n";
+      else if (b.kind == KernelBinding::Softmax)
+        os << "inline int kernel" << b.index << "(float* arg0 /*x, in place*/, void* stream = nullptr) {\n"
+           << "  return kcg_softmax_f32(arg0, " << b.count / b.rowLength << ", " << b.rowLength << ", stream);\n}\n\n";
+      else
+        os << "inline int kernel" << b.index
+           << "(const float* arg0 /*A*/, const float* arg1 /*B*/, float* arg2 /*C*/, void* stream = nullptr) {\n"
+           << "  return kcg_batched_matmul_f32(arg0, " << b.transA << ", arg1, " << b.transB << ", arg2, " << b.batch
+           << ", " << b.M << ", " << b.N << ", " << b.K << ", stream);\n}\n\n";
+      continue;
+    }
     os << "// " << b.funcName << " -> " << b.launch.kernel << "\n"
        << "// grid dims:(" << b.launch.grid[0] << ", " << b.launch.grid[1] << ", " << b.launch.grid[2]
        << "), block dims:(" << b.launch.block[0] << ", " << b.launch.block[1] << ", " << b.launch.block[2]
@@ -268,6 +418,14 @@ int HIPLaunch(const KernelBinding &b, const std::vector<void *> &p, void *stream
   if (b.kind == KernelBinding::Gemm)
     return kcg_gemm_f32(static_cast<const float *>(p[0]), static_cast<const float *>(p[1]),
                         static_cast<float *>(p[2]), b.M, b.N, b.K, b.epilogue, &b.gemmSched, stream);
+  if (b.kind == KernelBinding::Relu)
+    return kcg_relu_f32(static_cast<const float *>(p[0]), static_cast<float *>(b.inPlace ? p[0] : p[1]), b.count,
+                        stream);
+  if (b.kind == KernelBinding::Softmax)
+    return kcg_softmax_f32(static_cast<float *>(p[0]), b.count / b.rowLength, b.rowLength, stream);
+  if (b.kind == KernelBinding::BatchedMatmul)
+    return kcg_batched_matmul_f32(static_cast<const float *>(p[0]), b.transA, static_cast<const float *>(p[1]),
+                                  b.transB, static_cast<float *>(p[2]), b.batch, b.M, b.N, b.K, stream);
   if (b.dtype == KCG_BF16)
     return kcg_fmha_bf16(static_cast<const uint16_t *>(p[0]), static_cast<const uint16_t *>(p[1]),
                          static_cast<const uint16_t *>(p[2]), p[3], KCG_BF16, b.B, b.H, b.S, b.D, b.scale,

@@ -34,8 +34,10 @@ std::string scheduleText(const KernelBinding &b) {
   char buf[64];
   if (b.kind == KernelBinding::Gemm)
     snprintf(buf, sizeof buf, "%dx%dx%d", b.gemmSched.block_m, b.gemmSched.block_n, b.gemmSched.block_k);
-  else
+  else if (b.kind == KernelBinding::Fmha)
     snprintf(buf, sizeof buf, "br%d bc%d", b.fmhaSched.br, b.fmhaSched.bc);
+  else
+    snprintf(buf, sizeof buf, "unfused");
   return buf;
 }
 
@@ -107,15 +109,8 @@ float HIPTimer::operator()(ir::ModuleOp &module) {
     t.func = b.funcName;
     t.kernel = b.launch.kernel;
     t.schedule = scheduleText(b);
-    std::vector<size_t> bytes;
+    const std::vector<size_t> &bytes = b.argBytes;
     const bool bf16 = b.kind == KernelBinding::Fmha && b.dtype == KCG_BF16;
-    if (b.kind == KernelBinding::Gemm) {
-      bytes = {static_cast<size_t>(b.M * b.K) * 4, static_cast<size_t>(b.K * b.N) * 4,
-               static_cast<size_t>(b.M * b.N) * 4};
-    } else {
-      const size_t n = static_cast<size_t>(b.B) * b.H * b.S * b.D * (bf16 ? 2 : 4);
-      bytes = {n, n, n, n};
-    }
     std::vector<void *> ptrs;
     for (size_t i = 0; i < bytes.size(); ++i) ptrs.push_back(buffer(i, bytes[i], bf16));
     bool allocated = true;

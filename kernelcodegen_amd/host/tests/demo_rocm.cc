@@ -8,6 +8,14 @@
 //                    the scheduled nest ("schedule <source> block_k <n> lds_stages <n>
 //                    vec_width <n>" is printed)
 //   demo_rocm fmha   B H S D causal(0|1) scale out.bin
+//   demo_rocm fmharef B H S D causal(0|1) scale out.bin    the reference's own attention table
+//                    (HdxBr = BrxBc = 8192, include/KernelCodeGen.h:38-41 there): Br 64 x Bc 128
+//                    at head dim 128, Br 128 x Bc 64 at head dim 64
+//   demo_rocm unfused attn B H S D out.bin     S = Q.K^T, R = Relu(S) into a buffer of its own,
+//                    P = Softmax(S), O = P.V: the score tensor has two users, the attention
+//                    pattern does not match, and the four calls are bound one kernel each to
+//                    the un-fused entry points; out.bin holds O followed by R
+//   demo_rocm unfused softmax ROWS N out.bin   a Softmax on its own, in place
 //   demo_rocm tune matmul M N K relu(0|1) out.bin
 //   demo_rocm tune fmha   B H S D causal(0|1) scale out.bin
 //
@@ -86,6 +94,60 @@ static int run(const KernelBinding &b, const std::vector<std::vector<float> *> &
   return 0;
 }
 
+// Runs every binding of a module in order.  One device buffer per distinct module-level
+// buffer (KernelBinding::buffers): `inputs` are uploaded, the others start as zeros;
+// `outputs` are written to outPath one after the other.
+static int runGraph(const std::vector<KernelBinding> &bindings,
+                    const std::vector<std::pair<ir::Value, std::vector<float> *>> &inputs,
+                    const std::vector<ir::Value> &outputs, const char *outPath) {
+  std::vector<std::pair<ir::Value, void *>> dev;
+  std::vector<size_t> bytes;
+  auto find = [&](ir::Value v) -> int {
+    for (size_t i = 0; i < dev.size(); ++i)
+      if (dev[i].first == v) return static_cast<int>(i);
+    return -1;
+  };
+  for (auto &b : bindings)
+    for (size_t i = 0; i < b.buffers.size(); ++i) {
+      if (find(b.buffers[i]) >= 0) continue;
+      void *d = nullptr;
+      HIP_OK(hipMalloc(&d, b.argBytes[i]));
+      HIP_OK(hipMemset(d, 0, b.argBytes[i]));
+      dev.emplace_back(b.buffers[i], d);
+      bytes.push_back(b.argBytes[i]);
+    }
+  for (auto &in : inputs) {
+    const int at = find(in.first);
+    if (at < 0 || bytes[at] != in.second->size() * sizeof(float)) return 6;
+    HIP_OK(hipMemcpy(dev[at].second, in.second->data(), bytes[at], hipMemcpyHostToDevice));
+  }
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  for (auto &b : bindings) {
+    std::vector<void *> p;
+    for (auto v : b.buffers) p.push_back(dev[find(v)].second);
+    const int st = HIPLaunch(b, p, stream);
+    if (st != KCG_OK) {
+      std::fprintf(stderr, "launch of %s failed: %s\n", b.funcName.c_str(), kcg_status_str(st));
+      return 3;
+    }
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+  FILE *fp = std::fopen(outPath, "wb");
+  if (!fp) return 4;
+  for (auto v : outputs) {
+    const int at = find(v);
+    if (at < 0) return 6;
+    std::vector<float> host(bytes[at] / sizeof(float));
+    HIP_OK(hipMemcpy(host.data(), dev[at].second, bytes[at], hipMemcpyDeviceToHost));
+    std::fwrite(host.data(), sizeof(float), host.size(), fp);
+  }
+  std::fclose(fp);
+  for (auto &d : dev) HIP_OK(hipFree(d.second));
+  HIP_OK(hipStreamDestroy(stream));
+  return 0;
+}
+
 int main(int argc, char **argv) {
   if (argc < 2) {
     std::fprintf(stderr, "usage: demo_rocm [tune] matmul M N K relu out | demo_rocm [tune] fmha B H S D causal scale out\n");
@@ -148,6 +210,56 @@ int main(int argc, char **argv) {
     fill_uniform(a, kSeed, 0);
     fill_uniform(b, kSeed, 1);
     return run(bindings[0], {&a, &b}, static_cast<size_t>(m * n), argv[6]);
+  }
+  if (mode == "unfused" && argc == 8 && std::string(argv[2]) == "attn") {
+    const int64_t bsz = std::atoll(argv[3]), h = std::atoll(argv[4]), s = std::atoll(argv[5]), d = std::atoll(argv[6]);
+    auto &graph = generator.createGraph("unfused_attn_demo");
+    std::vector<int64_t> shape{bsz, h, s, d};
+    auto Q = graph.create<PlaceHolder>(shape, std::string{"float32"});
+    auto K = graph.create<PlaceHolder>(shape, std::string{"float32"});
+    auto V = graph.create<PlaceHolder>(shape, std::string{"float32"});
+    auto S = graph.create<BatchedMatmul>(Q, Layout::rowMajor, K, Layout::colMajor);
+    auto R = graph.create<Relu>(S, MemorySpace::global);   // a second reader of the scores
+    auto P = graph.create<Softmax>(S, -1, MemorySpace::inplace);
+    auto O = graph.create<BatchedMatmul>(P, Layout::rowMajor, V, Layout::rowMajor);
+    auto module = generator.optimize(graph);
+    auto bindings = generator.bind(module);
+    std::printf("bindings %zu:", bindings.size());
+    for (auto &b : bindings) std::printf(" %s", b.entry.c_str());
+    std::printf("\n%s", generator.codegen(module).c_str());
+    if (bindings.size() != 4) return 5;
+    // the module optimize() returned is a copy: the buffers are named through its own values
+    const size_t count = static_cast<size_t>(bsz * h * s * d);
+    std::vector<float> q(count), kk(count), v(count);
+    fill_uniform(q, kSeed, 0);
+    fill_uniform(kk, kSeed, 1);
+    fill_uniform(v, kSeed, 2);
+    (void)Q; (void)K; (void)V; (void)R; (void)O;
+    // binding 0 = Q.K^T (A, B, C), binding 1 = Relu (x, y), binding 3 = P.V (A, B, C)
+    return runGraph(bindings,
+                    {{bindings[0].buffers[0], &q}, {bindings[0].buffers[1], &kk}, {bindings[3].buffers[1], &v}},
+                    {bindings[3].buffers[2], bindings[1].buffers[1]}, argv[7]);
+  }
+  if (mode == "unfused" && argc == 6 && std::string(argv[2]) == "softmax") {
+    const int64_t rows = std::atoll(argv[3]), n = std::atoll(argv[4]);
+    auto &graph = generator.createGraph("softmax_demo");
+    auto X = graph.create<PlaceHolder>(std::vector<int64_t>{rows, n}, std::string{"float32"});
+    graph.create<Softmax>(X, -1, MemorySpace::inplace);
+    auto module = generator.optimize(graph);
+    auto bindings = generator.bind(module);
+    std::printf("bindings %zu:", bindings.size());
+    for (auto &b : bindings) std::printf(" %s", b.entry.c_str());
+    std::printf("\n%s", generator.codegen(module).c_str());
+    if (bindings.size() != 1) return 5;
+    std::vector<float> x(static_cast<size_t>(rows * n));
+    fill_uniform(x, kSeed, 0);
+    for (auto &e : x) e *= 4.0f;
+    return runGraph(bindings, {{bindings[0].buffers[0], &x}}, {bindings[0].buffers[0]}, argv[5]);
+  }
+  if (mode == "fmharef" && argc == 9) {
+    // the reference's own table: 128 threads, Br = 8192 / Hd, Bc = 8192 / Br
+    generator.fmhaConfigs = {{{"BLOCK_SIZE", 128}, {"HdxBr", 8192}, {"BrxBc", 8192}, {"WARP_SIZE", 32}}};
+    mode = "fmha";
   }
   if (mode == "fmha" && argc == 9) {
     const int64_t bsz = std::atoll(argv[2]), h = std::atoll(argv[3]), s = std::atoll(argv[4]), d = std::atoll(argv[5]);

@@ -868,6 +868,108 @@ static void test_facade_flash_attention_demo() {
   CHECK(contains(g2.codegen(module2), "kcg_fmha_bf16(arg0, arg1, arg2, arg3, KCG_BF16, 4, 32, 4096, 128, 1.0f, 1, &sched, stream)"));
 }
 
+// Graphs no pattern matches: every call is bound to its un-fused kernel, in module order,
+// and the bindings name the module-level buffers their pointers stand for.
+static void test_unfused_binding() {
+  KernelCodeGenerator generator("ROCm");
+  generator.setLogMode(Log::Release);
+  auto &graph = generator.createGraph("unfused");
+  std::vector<int64_t> shp{2, 3, 96, 64};
+  auto Q = graph.create<PlaceHolder>(shp, std::string{"float32"});
+  auto K = graph.create<PlaceHolder>(shp, std::string{"float32"});
+  auto V = graph.create<PlaceHolder>(shp, std::string{"float32"});
+  auto S = graph.create<BatchedMatmul>(Q, Layout::rowMajor, K, Layout::colMajor);
+  graph.create<Relu>(S, MemorySpace::global);   // second reader of the scores, own result buffer
+  auto P = graph.create<Softmax>(S, -1, MemorySpace::inplace);
+  graph.create<BatchedMatmul>(P, Layout::rowMajor, V, Layout::rowMajor);
+  auto module = generator.optimize(graph);
+  CHECK(verify(module.get()).empty());
+  auto b = generator.bind(module);
+  CHECK(b.size() == 4);
+  if (b.size() == 4) {
+    CHECK(b[0].kind == KernelBinding::BatchedMatmul && b[0].entry == "kcg_batched_matmul_f32");
+    CHECK(b[0].batch == 6 && b[0].M == 96 && b[0].N == 96 && b[0].K == 64 && b[0].transA == 0 && b[0].transB == 1);
+    CHECK(b[0].argBytes == (std::vector<size_t>{6 * 96 * 64 * 4, 6 * 96 * 64 * 4, 6 * 96 * 96 * 4}));
+    CHECK(b[1].kind == KernelBinding::Relu && !b[1].inPlace && b[1].count == 6 * 96 * 96 && b[1].argNames.size() == 2);
+    CHECK(b[2].kind == KernelBinding::Softmax && b[2].inPlace && b[2].rowLength == 96 && b[2].count == 6 * 96 * 96);
+    CHECK(b[3].kind == KernelBinding::BatchedMatmul && b[3].transA == 0 && b[3].transB == 0 && b[3].K == 96 && b[3].N == 64);
+    for (int i = 0; i < 4; ++i) CHECK(b[i].index == i && b[i].buffers.size() == b[i].argNames.size());
+    // the scores: written by the first product, read by Relu, rewritten in place by Softmax,
+    // and -- through Softmax's result -- the left operand of the second product
+    CHECK(b[0].buffers[2] == b[1].buffers[0] && b[0].buffers[2] == b[2].buffers[0] && b[0].buffers[2] == b[3].buffers[0]);
+    CHECK(b[1].buffers[1] != b[1].buffers[0]);                       // Relu's own result
+    CHECK(b[0].buffers[0] != b[0].buffers[1] && b[3].buffers[1] != b[0].buffers[1]);   // Q, K, V apart
+    CHECK(b[0].buffers[2].getDefiningOp() && b[0].buffers[2].getDefiningOp()->kind == OpKind::Alloc);
+  }
+  const std::string src = generator.codegen(module);
+  CHECK(contains(src, "namespace unfused {"));
+  CHECK(contains(src, "return kcg_batched_matmul_f32(arg0, 0, arg1, 1, arg2, 6, 96, 96, 64, stream);"));
+  CHECK(contains(src, "inline int kernel1(const float* arg0 /*x*/, float* arg1 /*y*/, void* stream = nullptr)"));
+  CHECK(contains(src, "return kcg_relu_f32(arg0, arg1, 55296, stream);"));
+  CHECK(contains(src, "return kcg_softmax_f32(arg0, 576, 96, stream);"));
+  CHECK(contains(src, "return kcg_batched_matmul_f32(arg0, 0, arg1, 0, arg2, 6, 96, 64, 96, stream);"));
+  // a Softmax on its own, an in-place Relu on its own
+  KernelCodeGenerator g2;
+  g2.setLogMode(Log::Release);
+  auto &lone = g2.createGraph("lone");
+  auto X = lone.create<PlaceHolder>(std::vector<int64_t>{40, 1000}, std::string{"float32"});
+  auto Y = lone.create<Softmax>(X, -1, MemorySpace::inplace);
+  lone.create<Relu>(Y, MemorySpace::inplace);
+  auto m2 = g2.optimize(lone);
+  auto b2 = g2.bind(m2);
+  CHECK(b2.size() == 2);
+  if (b2.size() == 2) {
+    CHECK(b2[0].kind == KernelBinding::Softmax && b2[0].rowLength == 1000 && b2[0].count == 40000);
+    CHECK(b2[1].kind == KernelBinding::Relu && b2[1].inPlace && b2[1].argNames.size() == 1);
+    CHECK(b2[0].buffers[0] == b2[1].buffers[0]);
+  }
+  CHECK(contains(g2.codegen(m2), "return kcg_relu_f32(arg0, arg0, 40000, stream);"));
+  // a trailing in-place Relu behind a Matmul still folds into the matmul's epilogue: one binding
+  KernelCodeGenerator g3;
+  g3.setLogMode(Log::Release);
+  auto &mm = g3.createGraph("mm");
+  auto A = mm.create<PlaceHolder>(std::vector<int64_t>{256, 64}, std::string{"float32"});
+  auto B = mm.create<PlaceHolder>(std::vector<int64_t>{64, 128}, std::string{"float32"});
+  auto C = mm.create<Matmul>(A, B, MemorySpace::global);
+  mm.create<Relu>(C, MemorySpace::inplace);
+  auto b3 = g3.bind(g3.optimize(mm));
+  CHECK(b3.size() == 1 && b3[0].kind == KernelBinding::Gemm && b3[0].epilogue == KCG_EPILOGUE_RELU);
+  // other element types have no un-fused kernel: reported and skipped
+  KernelCodeGenerator g4;
+  g4.setLogMode(Log::Release);
+  auto &half = g4.createGraph("half");
+  auto H = half.create<PlaceHolder>(std::vector<int64_t>{8, 64}, std::string{"float16"});
+  half.create<Softmax>(H, -1, MemorySpace::inplace);
+  std::vector<KernelBinding> b4;
+  quiet([&] { b4 = g4.bind(g4.optimize(half)); });
+  CHECK(b4.empty());
+}
+
+// The reference's own attention table (include/KernelCodeGen.h:38-41 there: 128 threads,
+// HdxBr = BrxBc = 8192) binds: Br 64 x Bc 128 at head dim 128, Br 128 x Bc 64 at head dim 64.
+static void test_reference_attention_table_binds() {
+  for (int hd : {128, 64}) {
+    KernelCodeGenerator generator("ROCm");
+    generator.setLogMode(Log::Release);
+    generator.fmhaConfigs = {{{"BLOCK_SIZE", 128}, {"HdxBr", 8192}, {"BrxBc", 8192}, {"WARP_SIZE", 32}}};
+    auto &graph = attention_graph(generator, 8, 32, 2048, hd);
+    auto module = generator.optimize(graph);
+    auto b = generator.bind(module);
+    CHECK(b.size() == 1);
+    if (b.size() != 1) continue;
+    CHECK(b[0].kind == KernelBinding::Fmha && b[0].fmhaSched.br == 8192 / hd && b[0].fmhaSched.bc == hd);
+    CHECK(b[0].launch.block[0] == (hd == 128 ? 128 : 256));       // two waves / four waves of 32 rows
+    CHECK(b[0].launch.grid[0] == 8 * 32 * (2048 / (8192 / hd)));
+    // and for bf16 operands
+    KernelCodeGenerator g2;
+    g2.setLogMode(Log::Release);
+    g2.fmhaConfigs = generator.fmhaConfigs;
+    auto &graph2 = attention_graph(g2, 2, 4, 512, hd, "bfloat16");
+    auto b2 = g2.bind(g2.optimize(graph2));
+    CHECK(b2.size() == 1 && b2[0].entry == "kcg_fmha_bf16" && b2[0].fmhaSched.br == 8192 / hd);
+  }
+}
+
 static void test_error_paths() {
   quiet([] {
     KernelCodeGenerator gen;
@@ -980,6 +1082,8 @@ int main() {
       {"schedule_drives_binding", test_schedule_drives_binding},
       {"facade_config_search_and_reference_tile", test_facade_config_search_and_reference_tile},
       {"facade_flash_attention_demo", test_facade_flash_attention_demo},
+      {"unfused_binding", test_unfused_binding},
+      {"reference_attention_table_binds", test_reference_attention_table_binds},
       {"error_paths", test_error_paths},
       {"verify_and_clone", test_verify_and_clone},
       {"builders_outer_product_set_buffer", test_builders_outer_product_set_buffer},

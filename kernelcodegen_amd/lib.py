@@ -51,6 +51,8 @@ SYMBOLS = {
     "kcg_gemm_f32_ws_bytes": (ctypes.c_int64, [_i64, _i64, _i64, ctypes.POINTER(GemmSched)]),
     "kcg_gemm_f32_ws": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_int,
                                        ctypes.POINTER(GemmSched), _vp, _i64, _vp]),
+    "kcg_gemm_f32_ws_query": (ctypes.c_int, [_i64, _i64, _i64, ctypes.POINTER(GemmSched), _i64,
+                                             ctypes.POINTER(LaunchInfo)]),
     "kcg_gemm_f32_noalloc": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_int,
                                             ctypes.POINTER(GemmSched), _vp]),
     "kcg_gemm_f32_query": (ctypes.c_int, [_i64, _i64, _i64, ctypes.POINTER(GemmSched),

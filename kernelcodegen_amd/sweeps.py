@@ -93,7 +93,11 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=Fal
         flops = 2.0 * M * N * K
         iters = max(3, min(50, int(2e12 / flops)))
         info = lib.LaunchInfo()
-        lib.check(L.kcg_gemm_f32_query(M, N, K, None, ctypes.byref(info)))
+        # (the geometry of the launches that are timed: with a workspace, the K-split pair)
+        if workspace:
+            lib.check(L.kcg_gemm_f32_ws_query(M, N, K, None, ws.numel() * 4, ctypes.byref(info)))
+        else:
+            lib.check(L.kcg_gemm_f32_query(M, N, K, None, ctypes.byref(info)))
         mine = _time(lambda: ops.matmul(A, B, relu=relu, out=C, workspace=ws), iters)
         split_bytes = ops.matmul_workspace_bytes(M, N, K) if workspace else 0
         if dump_dir:
@@ -112,11 +116,12 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=Fal
         tf = flops / mine / 1e9
         kernels = info.kernel.decode()
         geometry = "grid %d x %d threads, %d B LDS" % (info.grid[0], info.block[0], info.lds_bytes)
-        if info.launches == 2:
+        if info.launches == 2 and info.tail_rows:
             geometry += "; second launch %s on the last %d rows, grid %d x %d threads, %d B LDS" % (
                 info.tail_kernel.decode(), info.tail_rows, info.tail_grid[0], info.tail_block[0], info.tail_lds_bytes)
-        if split_bytes:
-            geometry += "; with the workspace lent: K-split plan, %d bytes of partial tiles and a second launch that adds them up" % split_bytes
+        elif info.launches == 2:
+            geometry += "; K-split plan with %d bytes of partial tiles, second launch %s adds them up, grid %d x %d threads" % (
+                split_bytes, info.tail_kernel.decode(), info.tail_grid[0], info.tail_block[0])
         print("Matrix size : \n --- M --- : %d\n --- N --- : %d\n --- K --- : %d\n" % (M, N, K))
         print("Occupancy: %.0f%%  (computed from the launch geometry: %s, %s)" % (
             computed_occupancy_percent(info), kernels, geometry))

@@ -294,12 +294,30 @@ def test_workspace_entry_points_check_their_arguments():
     assert L.kcg_gemm_f32_noalloc(fake, fake, fake, -1, 64, 64, 0, None, None) == 2
     assert L.kcg_gemm_f32_noalloc(fake, fake, fake, 64, 64, 64, 9, None, None) == 5
     assert L.kcg_gemm_f32_noalloc(fake, fake, fake, 66000, 128, 33000, 0, None, None) == 3
-    # 1536^3: 576 tiles = 2 x 256 + 64, the 64 in four pieces of 64 x 64 floats
+    # a negative GROUP_SIZE_M on a K-split shape is refused like kcg_gemm_f32 refuses it, before
+    # the split launch could number its tiles with it (status only: no device call is reached)
+    neg = lib.GemmSched(group_m=-1)
+    assert L.kcg_gemm_f32_ws(fake, fake, fake, 1536, 1536, 1536, 0, ctypes.byref(neg), fake, 1 << 26, None) == 4
+    assert L.kcg_gemm_f32_noalloc(fake, fake, fake, 1536, 1536, 1536, 0, ctypes.byref(neg), None) == 4
+    assert L.kcg_gemm_f32(fake, fake, fake, 1536, 1536, 1536, 0, ctypes.byref(neg), None) == 4
     assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 1536, None) == 64 * 4 * 64 * 64 * 4
     assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 256, None) == 0       # too little K to pay for a second launch
     assert L.kcg_gemm_f32_ws_bytes(4096, 4096, 4096, None) == 0      # the large tile, evenly filled
     assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 1540, None) == 0      # not whole slices
     assert L.kcg_gemm_f32_ws_bytes(0, 1536, 1536, None) == 0
+    # the launch pair of that plan, as the query entry point reports it
+    info = lib.LaunchInfo()
+    assert L.kcg_gemm_f32_ws_query(1536, 1536, 1536, None, 1 << 26, ctypes.byref(info)) == 0
+    assert info.launches == 2 and info.grid[0] == 512 + 64 * 4 and info.block[0] == 256
+    assert info.lds_bytes == 52224 and b"split" in info.kernel and b"reduce" in info.tail_kernel
+    assert info.tail_grid[0] == 64 * 4 and info.main_rows == 1536 and info.tail_rows == 0
+    plain = lib.LaunchInfo()
+    assert L.kcg_gemm_f32_ws_query(1536, 1536, 1536, None, 0, ctypes.byref(info)) == 0
+    assert L.kcg_gemm_f32_query(1536, 1536, 1536, None, ctypes.byref(plain)) == 0
+    assert bytes(info) == bytes(plain)           # no room for a plan: the answer of the plain query
+    assert L.kcg_gemm_f32_ws_query(1536, 1536, 1536, None, -1, ctypes.byref(info)) == 5
+    assert L.kcg_gemm_f32_ws_query(1536, 1536, 1536, ctypes.byref(neg), 1 << 26, ctypes.byref(info)) == 4
+    assert L.kcg_gemm_f32_ws_query(1536, 1536, 1536, None, 1 << 26, None) == 1
     fixed = lib.GemmSched(block_m=64, block_n=64, block_k=32, wave_m=32, wave_n=32)
     assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 1536, ctypes.byref(fixed)) == 0
     assert L.kcg_gemm_f32_ws_bytes(1536, 1536, 1536, ctypes.byref(lib.GemmSched(group_m=4))) == 64 * 4 * 64 * 64 * 4

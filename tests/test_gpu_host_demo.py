@@ -80,6 +80,53 @@ def test_flash_attention_demo(oracle, dev, tmp_path, causal):
     assert max(rel_err(got.reshape(B, H, S, D), ref)) < 1e-4
 
 
+@pytest.mark.parametrize("D,br,bc,threads", [(128, 64, 128, 128), (64, 128, 64, 256)])
+@pytest.mark.parametrize("causal", [0, 1])
+def test_reference_attention_table(oracle, dev, tmp_path, D, br, bc, threads, causal):
+    """The reference's own attention table (include/KernelCodeGen.h:38-41 there: HdxBr = BrxBc =
+    8192, src/Optimizer/Optimizer.cc:1136-1144) carried through the facade: Br 64 x Bc 128 at
+    head dim 128 (two waves of 32 query rows), Br 128 x Bc 64 at head dim 64."""
+    B, H, S = 2, 3, 320
+    scale = 0.125
+    got, text = _run(["fmharef", B, H, S, D, causal, scale], tmp_path)
+    assert "static const kcg_fmha_sched sched = {%d, %d};" % (br, bc) in text
+    assert "block dims:(%d, 1, 1)" % threads in text
+    Q, K, V = (inputs.uniform((B, H, S, D), SEED, i) for i in range(3))
+    ref = oracle.fmha(Q, K, V, scale=scale, causal=bool(causal), stable=True)
+    assert max(rel_err(got.reshape(B, H, S, D), ref)) < 1e-4
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 192, 64), (1, 2, 100, 128)])
+def test_unfused_graph(oracle, dev, tmp_path, shape):
+    """A graph the attention pattern rejects (the score tensor has a second reader,
+    src/Optimizer/Optimizer.cc:597-652 of the reference falls through): S = Q.K^T,
+    R = Relu(S) into its own buffer, P = Softmax(S) in place, O = P.V.  The host backend binds
+    the four calls to the un-fused kernels, one launcher each in module order, with S shared
+    between them; O and R against the oracle's operators chained the same way."""
+    B, H, S, D = shape
+    got, text = _run(["unfused", "attn", B, H, S, D], tmp_path)
+    assert "bindings 4: kcg_batched_matmul_f32 kcg_relu_f32 kcg_softmax_f32 kcg_batched_matmul_f32" in text
+    assert "return kcg_batched_matmul_f32(arg0, 0, arg1, 1, arg2, %d, %d, %d, %d, stream);" % (B * H, S, S, D) in text
+    assert "return kcg_softmax_f32(arg0, %d, %d, stream);" % (B * H * S, S) in text
+    Q, K, V = (inputs.uniform((B, H, S, D), SEED, i) for i in range(3))
+    scores = oracle.batched_matmul(Q, 0, K, 1)
+    R = oracle.relu(scores)
+    O = oracle.batched_matmul(oracle.softmax(scores), 0, V, 0)
+    n_o = B * H * S * D
+    assert got.size == n_o + B * H * S * S
+    assert max(rel_err(got[:n_o].reshape(B, H, S, D), O)) < 1e-4
+    assert max(rel_err(got[n_o:].reshape(B, H, S, S), R)) < 1e-4
+    assert np.array_equal(got[n_o:] == 0, R.reshape(-1) == 0)
+
+
+def test_lone_softmax(oracle, dev, tmp_path):
+    rows, n = 37, 1000
+    got, text = _run(["unfused", "softmax", rows, n], tmp_path)
+    assert "bindings 1: kcg_softmax_f32" in text and "namespace softmax_demo {" in text
+    x = inputs.uniform((rows, n), SEED, 0) * np.float32(4.0)
+    assert max(rel_err(got.reshape(rows, n), oracle.softmax(x))) < 1e-4
+
+
 def _trials(text):
     trials, best = [], None
     for line in text.splitlines():
