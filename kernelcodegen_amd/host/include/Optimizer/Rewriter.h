@@ -103,6 +103,17 @@ struct Rewriter {
   static ir::ForOp write(ir::OpHandle where, ir::Value src, ir::Value dst, const ir::AffineMap &map,
                          std::vector<ir::Value> operands, int64_t width);
 
+  // Copy loop from memory to memory, with no register buffer in between (gfx950 loads
+  // global memory straight into LDS; the reference stages through registers with read +
+  // write):
+  //   for i = 0 to count / width:  dst[dstMap(dstOperands, i)] .. +width) = src[srcMap(srcOperands, i)] .. +width)
+  // When dstMap has two dimensions more than there are dstOperands the `width` elements are
+  // stored one by one (an inner loop j < width binds the last dimension), which transposes
+  // on the way as write's scattering form does.
+  static ir::ForOp copy(ir::Value src, const ir::AffineMap &srcMap, std::vector<ir::Value> srcOperands,
+                        ir::Value dst, const ir::AffineMap &dstMap, std::vector<ir::Value> dstOperands,
+                        int64_t count, int64_t width, ir::ForOp compute_at, Position pos);
+
   // Every scalar load of `src` inside `scope` becomes a load of cached[map(operands)].
   static void cache_read(ir::ForOp scope, ir::Value src, ir::Value cached, const ir::AffineMap &map,
                          const std::vector<ir::Value> &operands);
@@ -133,6 +144,15 @@ struct Rewriter {
   // Returns {prologue loops, in-loop loops}.
   static std::vector<std::vector<ir::ForOp>> pipeline(std::vector<ir::ForOp> readBodys, ir::Value &buffer,
                                                       ir::ForOp compute_at);
+  // The same with a ring of `stages` copies (the reference hard-codes 2,
+  // src/Optimizer/Rewriter.cc:809-1180): the leading dimension becomes `stages`, the
+  // prologue fills the copies of the first stages - 1 iterations (result[0]: those loops,
+  // iteration-major), iteration i fetches iteration i + stages - 1 into copy
+  // (i + stages - 1) mod stages while one exists and every other access reads copy
+  // i mod stages.  One barrier per iteration (at its end) keeps such a ring coherent: the
+  // copy overwritten in iteration i is the one read in iteration i - 1.
+  static std::vector<std::vector<ir::ForOp>> pipeline(std::vector<ir::ForOp> readBodys, ir::Value &buffer,
+                                                      ir::ForOp compute_at, int stages);
   // Accesses to the double buffer `buffer` inside `forOp` switch to the other half.
   static void change_double_buffer(ir::ForOp forOp, ir::Value buffer);
   // Peels the last iteration: the loop stops one step early and a copy of its

@@ -109,8 +109,15 @@ ThreadOrg threadOrg(const std::map<std::string, int> &config) {
   o.blockDimX = o.bn / tn;
   const int64_t threads = o.blockDimY * o.blockDimX;
   o.warps = o.warp > 0 ? threads / o.warp : 0;
+  // waves as WAVE rows x columns of the block tile when WAVE_SIZE_M / WAVE_SIZE_N say so and
+  // account for every wave (256 x 128 in 64 x 64 wave tiles: 4 x 2), else 2 x (warps / 2)
   o.warpOrg[0] = 2;
   o.warpOrg[1] = o.warps / 2;
+  const int64_t wm = cfg("WAVE_SIZE_M", 0), wn = cfg("WAVE_SIZE_N", 0);
+  if (wm > 0 && wn > 0 && o.bm % wm == 0 && o.bn % wn == 0 && (o.bm / wm) * (o.bn / wn) == o.warps) {
+    o.warpOrg[0] = o.bm / wm;
+    o.warpOrg[1] = o.bn / wn;
+  }
   o.threadOrg[0] = 8;
   o.threadOrg[1] = o.warp / 8;
   const int64_t strideA = o.warpOrg[1] > 0 ? (o.warps / o.warpOrg[1]) * o.threadOrg[0] : 0;
@@ -120,6 +127,7 @@ ThreadOrg threadOrg(const std::map<std::string, int> &config) {
   o.ldgA = threads > 0 ? o.bk * o.bm / threads : 0;
   o.ldgB = threads > 0 ? o.bk * o.bn / threads : 0;
   o.consistent = o.warps >= 2 && o.warps % 2 == 0 && o.warp % 8 == 0 && threads % o.warp == 0 &&
+                 o.warpOrg[0] > 0 && o.warpOrg[1] > 0 && o.warpOrg[0] * o.warpOrg[1] == o.warps &&
                  o.fragA == tm && o.fragB == tn && o.width > 0 && o.fragA % o.width == 0 &&
                  o.fragB % o.width == 0 && o.ldgA >= o.width && o.ldgA % o.width == 0 && o.ldgB >= o.width &&
                  o.ldgB % o.width == 0 && o.bk % o.width == 0 && o.bn % o.width == 0 &&
@@ -226,7 +234,64 @@ void MatmulOptimizer::applyOptimzer(ModuleOp &module) {
     if (detail >= 1 && !org.consistent)
       std::cerr << "MatmulOptimizer: the staged schedule needs BLOCK_SIZE = 16 x THREAD_SIZE and whole warps; "
                    "keeping the tiled nest\n";
-    if (detail >= 1 && org.consistent && k_axes.size() == 2) {
+    if (detail == 3 && org.consistent && k_axes.size() == 2) {
+      // The direct-load form: global -> shared with no register tile in between, the shared
+      // tiles a ring of three copies along k_outer (two slices in flight while one is
+      // consumed), one barrier per slice.  This is the nest of the library's default matmul
+      // kernel; the reference's recipe (staged through registers, two copies) is detail 1 / 2.
+      ForOp k_outer = k_axes[0], k_inner = k_axes[1];
+      const int width = static_cast<int>(org.width);
+      const MemoryBuffer &buf = matmulBuffers[matmul];
+      const DType elemA = buf.A.getMemRefType().elem, elemB = buf.B.getMemRefType().elem;
+      Value fragB = Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {org.fragB}, elemB);
+      Value fragA = Rewriter::alloc_buffer(OpHandle(blockLevel.op), MemorySpace::local, {org.fragA}, elemA);
+      Value smB = Rewriter::alloc_buffer(OpHandle(gridLevel.op), MemorySpace::shared, {org.bk, org.bn}, elemB);
+      Value smA = Rewriter::alloc_buffer(OpHandle(gridLevel.op), MemorySpace::shared, {org.bk, org.bm}, elemA);
+      auto blockIdx = Rewriter::getParallelIdx(gridLevel);
+      auto threadIdx = Rewriter::getParallelIdx(blockLevel);
+      ForOp copyA = Rewriter::copy(buf.A, getAffineMap("loadTileA"),
+                                   {threadIdx[0], threadIdx[1], blockIdx[0], k_outer.getInductionVar()}, smA,
+                                   getAffineMap("storeTileA"), {threadIdx[0], threadIdx[1]}, org.ldgA, width, k_outer,
+                                   Position::begin);
+      ForOp copyB = Rewriter::copy(buf.B, getAffineMap("loadTileB"),
+                                   {threadIdx[0], threadIdx[1], k_outer.getInductionVar(), blockIdx[1]}, smB,
+                                   getAffineMap("storeTileB"), {threadIdx[0], threadIdx[1]}, org.ldgB, width, copyA,
+                                   Position::after);
+      DUMP(module);
+      ForOp loadFragA = Rewriter::read(smA, fragA, getAffineMap("loadFragA"),
+                                       {threadIdx[0], threadIdx[1], k_inner.getInductionVar()}, width, k_inner,
+                                       Position::begin);
+      Rewriter::read(smB, fragB, getAffineMap("loadFragB"), {threadIdx[0], threadIdx[1], k_inner.getInductionVar()},
+                     width, loadFragA, Position::after);
+      Rewriter::cache_read(k_inner, buf.A, fragA, getAffineMap("cacheReadA"), {m_inner.getInductionVar()});
+      Rewriter::cache_read(k_inner, buf.B, fragB, getAffineMap("cacheReadB"), {n_inner.getInductionVar()});
+      DUMP(module);
+      auto writeC = Rewriter::get_write(blockLevel, buf.C);
+      if (writeC.size() == 1 && writeC[0].size() == 2) {
+        auto m_inner_axes = Rewriter::split(writeC[0][0], 2, {width});
+        auto n_inner_axes = Rewriter::split(writeC[0][1], 2, {width});
+        ForOp m_inner_0 = m_inner_axes[0], m_inner_1 = m_inner_axes[1];
+        ForOp n_inner_0 = n_inner_axes[0], n_inner_1 = n_inner_axes[1];
+        Rewriter::reorder({m_inner_0, n_inner_0, m_inner_1, n_inner_1});
+        Rewriter::cache_write(m_inner_0, buf.C, tileC, getAffineMap("cacheWriteC"),
+                              {threadIdx[0], threadIdx[1], blockIdx[0], blockIdx[1], m_inner_0.getInductionVar(),
+                               n_inner_0.getInductionVar(), m_inner_1.getInductionVar(),
+                               n_inner_1.getInductionVar()});
+        Rewriter::vectorize(n_inner_1, width);
+        DUMP(module);
+      }
+      constexpr int kStages = 3;
+      Rewriter::pipeline({copyB}, smB, k_outer, kStages);
+      Rewriter::pipeline({copyA}, smA, k_outer, kStages);
+      // the slices of the prologue are published before the first one is read, and every
+      // iteration ends with the barrier that lets the next one overwrite the copy just read
+      Rewriter::barrier(k_outer, Position::before);
+      Rewriter::barrier(k_outer, Position::end);
+      DUMP(module);
+      Rewriter::take_off_true_if(module);
+      Rewriter::delete_false_if(module);
+      matmul.setAttr("kcg.schedule", "direct");
+    } else if (detail >= 1 && org.consistent && k_axes.size() == 2) {
       ForOp k_outer = k_axes[0], k_inner = k_axes[1];
       const int width = static_cast<int>(org.width);
       const MemoryBuffer &buf = matmulBuffers[matmul];

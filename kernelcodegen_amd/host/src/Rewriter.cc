@@ -426,6 +426,39 @@ ForOp Rewriter::write(OpHandle where, Value src, Value dst, const AffineMap &map
   return ForOp(loop);
 }
 
+ForOp Rewriter::copy(Value src, const AffineMap &srcMap, std::vector<Value> srcOperands, Value dst,
+                     const AffineMap &dstMap, std::vector<Value> dstOperands, int64_t count, int64_t width,
+                     ForOp compute_at, Position pos) {
+  if (!src || !dst || width <= 0 || count <= 0 || count % width != 0) {
+    std::cerr << "copy: needs two memrefs and a count that is a multiple of the width\n";
+    return ForOp();
+  }
+  Op *loop = placeLoop(compute_at, pos, makeFor(0, count / width, 1));
+  loop->pushBack(makeYield());
+  Op *yield = loop->lastOp();
+  const bool scatter = dstMap.numDims - static_cast<int>(dstOperands.size()) == 2;
+  srcOperands.push_back(loop->arg(0));
+  dstOperands.push_back(loop->arg(0));
+  if (!scatter) {
+    Op *ld = yield->insertBefore(makeVectorLoad(src, {}, static_cast<int>(width)));
+    ld->indices = materialize(srcMap, srcOperands, ld);
+    Op *st = yield->insertBefore(makeVectorStore(ld->result(), dst, {}, static_cast<int>(width)));
+    st->indices = materialize(dstMap, dstOperands, st);
+    return ForOp(loop);
+  }
+  // element j of the vector: the source's last subscript + j
+  Op *inner = yield->insertBefore(makeFor(0, width, 1));
+  inner->pushBack(makeYield());
+  Op *iy = inner->lastOp();
+  dstOperands.push_back(inner->arg(0));
+  Op *ld = iy->insertBefore(makeVectorLoad(src, {}, 1));
+  ld->indices = materialize(srcMap, srcOperands, ld);
+  ld->indices.back().add(inner->arg(0), 1);
+  Op *st = iy->insertBefore(makeVectorStore(ld->result(), dst, {}, 1));
+  st->indices = materialize(dstMap, dstOperands, st);
+  return ForOp(loop);
+}
+
 void Rewriter::cache_read(ForOp scope, Value src, Value cached, const AffineMap &map,
                           const std::vector<Value> &operands) {
   std::vector<Op *> loads;
@@ -521,15 +554,74 @@ void foldConstantApplies(Op *root) {
   }
 }
 
-// (iv floordiv step + offset) mod 2 as an index value computed right before `user`
-LinExpr halfSelector(Op *user, Value iv, int64_t step, int64_t offset) {
+// (iv floordiv step + offset) mod copies as an index value computed right before `user`
+LinExpr halfSelector(Op *user, Value iv, int64_t step, int64_t offset, int64_t copies = 2) {
   LinExpr q(iv);
   if (step != 1) q = LinExpr(user->insertBefore(makeApplyFloorDiv(LinExpr(iv), step))->result());
   q.constant += offset;
-  return LinExpr(user->insertBefore(makeApplyMod(q, 2))->result());
+  return LinExpr(user->insertBefore(makeApplyMod(q, copies))->result());
 }
 
 }  // namespace
+
+std::vector<std::vector<ForOp>> Rewriter::pipeline(std::vector<ForOp> readBodys, Value &buffer, ForOp compute_at,
+                                                   int stages) {
+  if (stages == 2) return pipeline(std::move(readBodys), buffer, compute_at);
+  std::vector<std::vector<ForOp>> results;
+  Op *def = buffer ? buffer.getDefiningOp() : nullptr;
+  if (!def || def->kind != OpKind::Alloc || readBodys.empty() || stages < 2) {
+    std::cerr << "pipeline: the buffer must come from memref.alloc, there must be a loop that fills it, and a ring "
+                 "has at least two copies\n";
+    return results;
+  }
+  for (auto r : readBodys)
+    if (!compute_at->isAncestorOf(r.op)) {
+      std::cerr << "pipeline: the filling loops must be inside the loop they are pipelined along\n";
+      return results;
+    }
+  Op *loop = compute_at.op;
+  Value iv = compute_at.getInductionVar();
+  const int64_t step = loop->step, lb = loop->lb, ub = loop->ub;
+  if (lb != 0) {
+    std::cerr << "pipeline: the ring is indexed by iv floordiv step, the loop must start at 0\n";
+    return results;
+  }
+  // 1. the ring
+  MemRefType t = buffer.getMemRefType();
+  t.shape.insert(t.shape.begin(), stages);
+  Value ring = def->insertBefore(makeAlloc(t))->result();
+  // 2. prologue: the copies of iterations 0 .. stages - 2, as far as the loop has them
+  std::vector<ForOp> prologue;
+  for (int s = 0; s + 1 < stages && lb + s * step < ub; ++s)
+    for (auto r : readBodys) {
+      Op *cp = loop->insertBefore(clone(r.op));
+      replaceIndexUses(cp, iv, LinExpr(lb + s * step));
+      retarget(cp, buffer, ring, [s](Op *) { return LinExpr(static_cast<int64_t>(s)); });
+      foldConstantApplies(cp);
+      prologue.emplace_back(cp);
+    }
+  results.push_back(prologue);
+  results.push_back(readBodys);
+  // 3. in the loop: fetch iteration i + stages - 1 while there is one
+  LinExpr guard;  // ub - stages * step - iv >= 0
+  guard.add(iv, -1);
+  guard.constant = ub - stages * step;
+  Op *ifOp = loop->pushFront(makeIf({guard}));
+  for (auto r : readBodys) {
+    auto owned = r->unlink();
+    Op *moved = ifOp->pushBack(std::move(owned));
+    LinExpr ahead(iv);
+    ahead.constant = (stages - 1) * step;
+    replaceIndexUses(moved, iv, ahead);
+    retarget(moved, buffer, ring, [&](Op *user) { return halfSelector(user, iv, step, stages - 1, stages); });
+  }
+  // 4. every remaining access reads the copy of the current iteration
+  Op *scope = def->parent;
+  retarget(scope, buffer, ring, [&](Op *user) { return halfSelector(user, iv, step, 0, stages); });
+  def->erase();
+  buffer = ring;
+  return results;
+}
 
 std::vector<std::vector<ForOp>> Rewriter::pipeline(std::vector<ForOp> readBodys, Value &buffer, ForOp compute_at) {
   std::vector<std::vector<ForOp>> results;

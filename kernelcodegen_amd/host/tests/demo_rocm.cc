@@ -2,11 +2,14 @@
 // flows (test/test.cc:8-107 there) carried through to a launch on the device.
 //
 //   demo_rocm matmul M N K relu(0|1) out.bin
-//   demo_rocm sched  M N K relu(0|1) detail(0|1|2) out.bin   the reference's 128 x 128 x 8 tile
-//                    with the staged (1) or pipelined (2) schedule built on the IR: the
-//                    binding reads block_k, the LDS buffer count and the vector width off
-//                    the scheduled nest ("schedule <source> block_k <n> lds_stages <n>
-//                    vec_width <n>" is printed)
+//   demo_rocm sched  M N K relu(0|1) detail(0|1|2|3) out.bin   the reference's 128 x 128 x 8 tile
+//                    with the staged (1), pipelined (2) or direct-load (3: no register tile,
+//                    a ring of three shared copies) schedule built on the IR: the binding
+//                    reads block_k, the LDS buffer count and the vector width off the
+//                    scheduled nest ("schedule <source> block_k <n> lds_stages <n> vec_width
+//                    <n>" is printed)
+//   demo_rocm sched256 M N K relu detail out.bin   the same on the library's default tile,
+//                    256 x 128 x 16 with eight waves of 64 x 64
 //   demo_rocm fmha   B H S D causal(0|1) scale out.bin
 //   demo_rocm fmharef B H S D causal(0|1) scale out.bin    the reference's own attention table
 //                    (HdxBr = BrxBc = 8192, include/KernelCodeGen.h:38-41 there): Br 64 x Bc 128
@@ -181,11 +184,13 @@ int main(int argc, char **argv) {
     }
   };
   std::string mode = argv[1];
-  if (mode == "sched" && argc == 8) {
+  if ((mode == "sched" || mode == "sched256") && argc == 8) {
     const int detail = std::atoi(argv[6]);
-    generator.matmulConfigs = {{{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 8}, {"GROUP_SIZE_M", 8},
-                                {"THREAD_SIZE_M", 8}, {"THREAD_SIZE_N", 8}, {"WAVE_SIZE_M", 64}, {"WAVE_SIZE_N", 64},
-                                {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64}, {"SCHEDULE_DETAIL", detail}}};
+    const bool big = mode == "sched256";
+    generator.matmulConfigs = {{{"BLOCK_SIZE_M", big ? 256 : 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", big ? 16 : 8},
+                                {"GROUP_SIZE_M", 8}, {"THREAD_SIZE_M", 8}, {"THREAD_SIZE_N", 8}, {"WAVE_SIZE_M", 64},
+                                {"WAVE_SIZE_N", 64}, {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64},
+                                {"SCHEDULE_DETAIL", detail}}};
     argv[6] = argv[7];
     --argc;
     mode = "matmul";

@@ -267,7 +267,8 @@ static void test_schedule_preserves_results() {
 // (src/Optimizer/Optimizer.cc:429-546), run by the interpreter with the threads of
 // a block in lock step: results must equal the naive nest bit for bit, for the
 // reference's 32-wide warps and for 64-wide waves.
-static void run_detailed_schedule(int detail, int warp, int64_t M, int64_t N, int64_t K, int bk, std::string *text) {
+static void run_detailed_schedule(int detail, int warp, int64_t M, int64_t N, int64_t K, int bk, std::string *text,
+                                  int bm = 128, int bn = 128, int waveM = 0, int waveN = 0) {
   std::vector<float> a(M * K), b(K * N);
   unsigned s = 777u + detail + warp;
   auto rnd = [&]() {
@@ -288,15 +289,17 @@ static void run_detailed_schedule(int detail, int warp, int64_t M, int64_t N, in
     }
   MatmulFixture f(M, N, K);
   MatmulOptimizer opt;
-  MatmulOptimizer::matmulConfig = {{"BLOCK_SIZE_M", 128}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", bk},
+  MatmulOptimizer::matmulConfig = {{"BLOCK_SIZE_M", bm}, {"BLOCK_SIZE_N", bn}, {"BLOCK_SIZE_K", bk},
                                    {"THREAD_SIZE_M", 8},  {"THREAD_SIZE_N", 8},   {"VECTORIZE_WIDTH", 4},
                                    {"WARP_SIZE", warp},   {"SCHEDULE_DETAIL", detail}};
+  if (waveM) MatmulOptimizer::matmulConfig["WAVE_SIZE_M"] = waveM;
+  if (waveN) MatmulOptimizer::matmulConfig["WAVE_SIZE_N"] = waveN;
   CHECK(opt.applicable(f.graph->module));
   opt.applyOptimzer(f.graph->module);
   const std::string problem = verify(f.graph->module.get());
   CHECK(problem.empty());
   if (!problem.empty()) std::fprintf(stderr, "    verify: %s\n", problem.c_str());
-  CHECK(f.func.getAttr("kcg.schedule") == (detail == 1 ? "staged" : "pipelined"));
+  CHECK(f.func.getAttr("kcg.schedule") == (detail == 1 ? "staged" : detail == 2 ? "pipelined" : "direct"));
   if (text) *text = f.graph->module.str();
   std::vector<float> c(M * N, -1.0f);
   Interpreter interp(f.graph->module);
@@ -347,6 +350,33 @@ static void test_pipelined_schedule() {
   CHECK(contains(text, "affine.loop = \"unroll\""));
   run_detailed_schedule(2, 64, 256, 128, 48, 8, nullptr);
   run_detailed_schedule(2, 64, 128, 128, 64, 16, nullptr);
+}
+
+// SCHEDULE_DETAIL 3: global -> shared with no register tile, a ring of three copies, one
+// barrier per slice -- the nest of the library's direct-load kernels.
+static void test_direct_schedule() {
+  std::string text;
+  run_detailed_schedule(3, 64, 128, 256, 40, 8, &text);            // five slices through a ring of three
+  CHECK(contains(text, "memref<3x8x128xf32, 2>"));
+  CHECK(!contains(text, "memref<8x128xf32, 2>") && !contains(text, "memref<2x8x128xf32, 2>"));
+  CHECK(!contains(text, "memref<4xf32, 3>"));                       // no register tile between global and shared
+  CHECK(contains(text, "memref<8xf32, 3>"));                        // fragments only
+  CHECK(contains(text, "mod 3"));
+  CHECK(contains(text, "affine.if affine_set<(d0) : (-d0 + 16 >= 0)>"));   // k_outer + 3*8 <= 40
+  CHECK(count(text, "affine.if") == 2);                             // one guard per operand's fetch
+  CHECK(count(text, "gpu.barrier") == 2);                           // after the prologue, at the end of a slice
+  // prologue: slices 0 and 1 of A and of B; in the loop one copy loop each
+  CHECK(count(text, "affine.vector_load %arg1[") == 3);
+  CHECK(contains(text, "memref<128x256xf32, 1>, vector<4xf32>"));
+  run_detailed_schedule(3, 64, 256, 128, 8, 8, nullptr);             // a single slice: prologue only
+  run_detailed_schedule(3, 64, 128, 128, 16, 8, nullptr);            // two slices: nothing left to fetch in the loop
+  run_detailed_schedule(3, 64, 128, 128, 64, 16, nullptr);
+  // the library's default tile: 256 x 128 x 16, eight waves of 64 x 64 (four by two), 8 x 8 per lane
+  run_detailed_schedule(3, 64, 256, 256, 64, 16, &text, 256, 128, 64, 64);
+  CHECK(contains(text, "memref<3x16x256xf32, 2>") && contains(text, "memref<3x16x128xf32, 2>"));
+  CHECK(contains(text, "affine.parallel (%arg3, %arg4) = (0, 0) to (32, 16)") || contains(text, "to (32, 16)"));
+  run_detailed_schedule(1, 64, 256, 128, 32, 16, nullptr, 256, 128, 64, 64);   // the same organisation, staged
+  run_detailed_schedule(2, 64, 256, 128, 48, 16, nullptr, 256, 128, 64, 64);   // and pipelined
 }
 
 static void test_relu_softmax_batched_matmul_semantics() {
@@ -763,6 +793,39 @@ static void test_schedule_drives_binding() {
       CHECK(contains(pipelined.str(), "memref<2x8x128xf32, 2>"));
     }
   }
+  {  // direct: memref<3x8x128xf32, 2> rings -> the three-stage direct-load kernel, read off the nest
+    ir::ModuleOp direct;
+    auto [b, src] = bindWith(3, &direct);
+    CHECK(b.size() == 1);
+    if (b.size() == 1) {
+      CHECK(b[0].scheduleSource == "ir" && b[0].gemmSched.lds_stages == 3 && b[0].scheduleNote.empty());
+      CHECK(b[0].gemmSched.block_k == 8 && b[0].gemmSched.vec_width == 4);
+      CHECK(std::string(b[0].launch.kernel) == "gemm_f32_128x128x8_w2x2_dl");
+      CHECK(contains(direct.str(), "memref<3x8x128xf32, 2>"));
+      CHECK(contains(src, "lds stages 3") && contains(src, "from the scheduled loop nest"));
+      CHECK(contains(src, "sched = {128, 128, 8, 8, 64, 64, 4, 64, 3};"));
+    }
+  }
+  {  // the library's default tile staged the same way: 256 x 128 x 16, eight waves of 64 x 64
+    KernelCodeGenerator generator("ROCm");
+    generator.setLogMode(Log::Release);
+    generator.matmulConfigs = {{{"BLOCK_SIZE_M", 256}, {"BLOCK_SIZE_N", 128}, {"BLOCK_SIZE_K", 16}, {"GROUP_SIZE_M", 8},
+                                {"THREAD_SIZE_M", 8}, {"THREAD_SIZE_N", 8}, {"WAVE_SIZE_M", 64}, {"WAVE_SIZE_N", 64},
+                                {"VECTORIZE_WIDTH", 4}, {"WARP_SIZE", 64}, {"SCHEDULE_DETAIL", 3}}};
+    auto &graph = generator.createGraph("sched_demo");
+    auto A = graph.create<PlaceHolder>(std::vector<int64_t>{1024, 512}, std::string{"float32"});
+    auto B = graph.create<PlaceHolder>(std::vector<int64_t>{512, 768}, std::string{"float32"});
+    graph.create<Matmul>(A, B, MemorySpace::global);
+    auto module = generator.optimize(graph);
+    auto b = generator.bind(module);
+    CHECK(b.size() == 1);
+    if (b.size() == 1) {
+      CHECK(b[0].scheduleSource == "ir" && b[0].gemmSched.lds_stages == 3 && b[0].gemmSched.block_k == 16);
+      CHECK(contains(b[0].launch.kernel, "gemm_f32_256x128x16") && contains(b[0].launch.kernel, "_dl"));
+      CHECK(b[0].launch.block[0] == 512 && b[0].launch.grid[0] == 4 * 6);
+      CHECK(contains(module.str(), "memref<3x16x256xf32, 2>"));
+    }
+  }
   {  // the attributes must not contradict the nest
     FuncOp f = Analyzer::collectFunctions(pipelined, "Matmul_m")[0];
     f.setAttr("kcg.BLOCK_SIZE_K", "16");
@@ -1073,6 +1136,7 @@ int main() {
       {"schedule_preserves_results", test_schedule_preserves_results},
       {"staged_schedule", test_staged_schedule},
       {"pipelined_schedule", test_pipelined_schedule},
+      {"direct_schedule", test_direct_schedule},
       {"relu_softmax_batched_matmul_semantics", test_relu_softmax_batched_matmul_semantics},
       {"batched_matmul_layouts", test_batched_matmul_layouts},
       {"fmha_pattern_and_fusion", test_fmha_pattern_and_fusion},

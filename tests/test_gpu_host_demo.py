@@ -38,14 +38,14 @@ def test_matmul_demo(oracle, dev, tmp_path, shape, relu):
     assert max(rel_err(got.reshape(M, N), ref)) < 1e-4
 
 
-@pytest.mark.parametrize("detail,stages,source", [(0, 0, "attributes"), (1, 2, "ir"), (2, 2, "ir")])
+@pytest.mark.parametrize("detail,stages,source", [(0, 0, "attributes"), (1, 2, "ir"), (2, 2, "ir"), (3, 3, "ir")])
 @pytest.mark.parametrize("shape", [(512, 384, 256), (384, 640, 72), (300, 260, 72)])
 def test_schedule_selects_the_kernel(oracle, dev, tmp_path, shape, detail, stages, source):
-    """The reference's 128 x 128 x 8 tile with the staged (SCHEDULE_DETAIL 1) and pipelined
-    (2) schedules built on the IR: the binding reads block_k, the LDS buffer count and the
-    vector width off the scheduled nest (the shared tiles memref<[2x]8x128xf32, 2>, the
-    float4 accesses), which selects the double-buffered register-staged kernel instead of
-    the library's default three-stage direct-load ring; the launched result is the oracle's.
+    """The reference's 128 x 128 x 8 tile with the staged (SCHEDULE_DETAIL 1), pipelined (2) and
+    direct-load (3) schedules built on the IR: the binding reads block_k, the LDS buffer count
+    and the vector width off the scheduled nest (the shared tiles memref<[2x|3x]8x128xf32, 2>,
+    the float4 accesses): one or two copies select the double-buffered register-staged kernel,
+    a ring of three the direct-load kernel; the launched result is the oracle's.
     Extents the tile does not divide keep the naive nest at every SCHEDULE_DETAIL (the
     optimizer only stages whole tiles), so their schedule comes from the attributes."""
     M, N, K = shape
@@ -63,6 +63,25 @@ def test_schedule_selects_the_kernel(oracle, dev, tmp_path, shape, detail, stage
     assert "static const kcg_gemm_sched sched = {128, 128, 8, 8, 64, 64, 4, 64, %d};" % stages in text
     if detail == 1 and whole_tiles:
         assert "// note: the nest keeps one copy of each shared tile" in text
+    A = inputs.uniform((M, K), SEED, 0)
+    B = inputs.uniform((K, N), SEED, 1)
+    ref = oracle.relu(oracle.matmul(A, B))
+    assert max(rel_err(got.reshape(M, N), ref)) < 1e-4
+
+
+@pytest.mark.parametrize("shape", [(1024, 768, 512), (512, 256, 48)])
+def test_default_tile_scheduled_on_the_ir(oracle, dev, tmp_path, shape):
+    """The library's default tile (256 x 128 x 16, eight waves of 64 x 64) staged on the IR as a
+    direct-load ring of three (SCHEDULE_DETAIL 3): the binding reads the ring depth and BLOCK_SIZE_K
+    off memref<3x16x256xf32, 2> / memref<3x16x128xf32, 2> and launches the default kernel."""
+    M, N, K = shape
+    got, text = _run(["sched256", M, N, K, 1, 3], tmp_path)
+    m = [l for l in text.splitlines() if l.startswith("schedule ")]
+    assert len(m) == 1
+    f = m[0].split()
+    assert f[1] == "ir" and int(f[3]) == 16 and int(f[5]) == 3 and int(f[7]) == 4
+    assert f[9].startswith("gemm_f32_256x128x16") and "_dl" in f[9]
+    assert "static const kcg_gemm_sched sched = {256, 128, 16, 8, 64, 64, 4, 64, 3};" in text
     A = inputs.uniform((M, K), SEED, 0)
     B = inputs.uniform((K, N), SEED, 1)
     ref = oracle.relu(oracle.matmul(A, B))
