@@ -30,12 +30,12 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 
 # HBM bytes per launch (fetch + write).  NOT measured by this script: counters cannot be
 # read from inside the timed run, so these are the figures of separate rocprofv3 --pmc
-# FETCH_SIZE / --pmc WRITE_SIZE runs of kernelcodegen_amd/profile_kernels.py, each scaled by
+# FETCH_SIZE / --pmc WRITE_SIZE runs of profile_kernels.py, each scaled by
 # the same counter's reading for a 256 MiB copy, as recorded in the named profile files.
 TRAFFIC = {
-    "gemm_cfg1": (744663460, "profiles/gemm_f32_cfg1.md"),
-    "fmha_cfg3": (138053321, "profiles/fmha_f32_cfg3.md"),
-    "fmha_cfg4": (787606226, "profiles/fmha_bf16_cfg4.md"),
+    "gemm_cfg1": (743925920, "profiles/gemm_f32_cfg1.md"),
+    "fmha_cfg3": (137533632, "profiles/fmha_f32_cfg3.md"),
+    "fmha_cfg4": (788052280, "profiles/fmha_bf16_cfg4.md"),
 }
 
 

@@ -2,18 +2,23 @@
 """Runs one workload's kernel a few times, preceded by a plain device-to-device
 copy of known size, so that a profiler run over this script sees both:
 
-    rocprofv3 --kernel-trace --stats -d OUT -- python3 kernelcodegen_amd/profile_kernels.py --workload gemm_cfg1
-    rocprofv3 --pmc FETCH_SIZE -d OUT -- python3 kernelcodegen_amd/profile_kernels.py --workload gemm_cfg1
-    rocprofv3 --pmc WRITE_SIZE -d OUT -- python3 kernelcodegen_amd/profile_kernels.py --workload gemm_cfg1
+    rocprofv3 --kernel-trace --stats -d OUT -- python3 profile_kernels.py --workload gemm_cfg1
+    rocprofv3 --pmc FETCH_SIZE -d OUT -- python3 profile_kernels.py --workload gemm_cfg1
+    rocprofv3 --pmc WRITE_SIZE -d OUT -- python3 profile_kernels.py --workload gemm_cfg1
 
 The copy (COPY_MIB MiB read + COPY_MIB MiB written per launch) calibrates the
 FETCH_SIZE / WRITE_SIZE counters: the factor is bytes-known / counter-read.
+
+The workload's launches come in two groups: a settle phase (launches of the same call
+until --settle-ms of wall-clock time have passed, so that the shader clock has left its
+ramp; their number is printed) and then --iters launches.  A kernel trace holds both
+groups; the launches after the settle phase are the last --iters of the kernel.
 """
 import argparse
 import os
 import sys
 
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 COPY_MIB = 256
 
@@ -30,8 +35,9 @@ def main():
     ap.add_argument("--tile", default="",
                     help="matmul workloads only: BLOCK_M x BLOCK_N x BLOCK_K of the schedule, e.g. 256x128x32 "
                          "(default: the library's choice)")
-    ap.add_argument("--iters", type=int, default=200,
-                    help="launches of the workload (the first tens run on a ramping clock)")
+    ap.add_argument("--iters", type=int, default=200, help="launches of the workload after the settle phase")
+    ap.add_argument("--settle-ms", type=float, default=40.0,
+                    help="wall-clock time of the launches that precede them (0: none)")
     args = ap.parse_args()
 
     import numpy as np
@@ -87,10 +93,18 @@ def main():
             Q, K, V = (torch.from_numpy(c[k]).to(dev) for k in "QKV")
         O = torch.empty_like(Q)
         fn = lambda: ops.fmha(Q, K, V, scale=c["scale"], causal=c["causal"], out=O)
+    import time
+    settle = 0
+    t0 = time.perf_counter()
+    while args.settle_ms > 0 and (time.perf_counter() - t0) * 1e3 < args.settle_ms:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+        settle += 4
     for _ in range(args.iters):
         fn()
     torch.cuda.synchronize()
-    print("done", args.workload, args.iters)
+    print("done", args.workload, "settle launches", settle, "then", args.iters)
 
 
 if __name__ == "__main__":
