@@ -15,6 +15,7 @@ depend on how many warm-up steps the caller asks for.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
     python bench.py --sweep matmul [--max-dim D | --dims D1,MxNxK,...] [--relu] [--seeded] [--dump DIR] [--workspace]
     python bench.py --sweep fmha | --sweep ops [--shape B,H,S,D]
+    python bench.py --sweep fmha-variants      (after `make -C kernelcodegen_amd/csrc variants`)
 """
 import argparse
 import json
@@ -118,7 +119,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the attention workloads")
-    ap.add_argument("--sweep", choices=["matmul", "fmha", "ops"],
+    ap.add_argument("--sweep", choices=["matmul", "fmha", "ops", "fmha-variants"],
                     help="instead of the benchmark line, print a measurement sweep: the reference's "
                          "matmul size sweep in its output.log format, the attention shape grid, or the "
                          "un-fused operators against their rooflines (kernelcodegen_amd/sweeps.py)")
@@ -155,6 +156,8 @@ def main():
                            for d in args.dims.split(",")] if args.dims else None)
         elif args.sweep == "fmha":
             sweeps.fmha()
+        elif args.sweep == "fmha-variants":
+            sweeps.fmha_variants()
         else:
             sweeps.ops_chain(tuple(int(x) for x in args.shape.split(",")))
         return

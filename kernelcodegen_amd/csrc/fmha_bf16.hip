@@ -499,6 +499,19 @@ __global__ __launch_bounds__(64 * WAVES, (QT == 1 && WAVES > 2 ? 2 : 1)) void fm
 //    pair, then the next work item, possibly of another head -- follow each other in one
 //    stream, so the pipeline is filled once per workgroup; the Q rows of the next block
 //    are requested right after the last S of the current one.
+//
+// Build-time experiment switches (all off in the library; `make variants` builds one library
+// per switch, `bench.py --sweep fmha-variants` times them against the default in one job).
+// Each is a lever on the causal sweep that was built, measured and not adopted:
+//   KCG_FMHA_EXP_ALL_PAIRS      waves also compute the diagonal tiles that lie wholly above
+//                               their rows (every score masked) instead of skipping them:
+//                               the tile loop then has no causal control flow at all.
+//   KCG_FMHA_EXP_LO_DESCENDING  the short block of a causal pair sweeps its tiles from the
+//                               diagonal down to tile 0, which puts all workgroups of a head
+//                               on the same K/V tile at the same time during that pass.
+//   KCG_FMHA_EXP_STAGE_O        the O rows of a pass leave through a 2 KiB LDS staging area per
+//                               wave as 64-byte row pieces (16 cache lines per store
+//                               instruction instead of 32 with 16 bytes each).
 template <int D>
 struct FmhaPpTile {
   static constexpr int kWaves = 8;
@@ -513,7 +526,13 @@ struct FmhaPpTile {
   static constexpr int kAhead = 3;               // tiles requested ahead of the one in use
   static constexpr int kRingK = 4;
   static constexpr int kRingV = 5;
-  static constexpr int kLdsBytes = (kRingK + kRingV) * kTile * 2;
+  static constexpr int kRingBytes = (kRingK + kRingV) * kTile * 2;
+#ifdef KCG_FMHA_EXP_STAGE_O
+  static constexpr int kStageBytes = 2048;       // per wave
+  static constexpr int kLdsBytes = kRingBytes + kWaves * kStageBytes;
+#else
+  static constexpr int kLdsBytes = kRingBytes;
+#endif
   static constexpr int kDTiles = D / 32;
   static constexpr int kDSteps = D / 16;
   static constexpr int kPvMfmas = 4 * kDTiles;   // MFMAs of O += P.V per tile
@@ -560,6 +579,12 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
   struct Pass {
     int item, pass, npass, bh, block, nt;
   };
+  // K/V tile that step `idx` of a pass works on
+#ifdef KCG_FMHA_EXP_LO_DESCENDING
+  auto tile_of = [&](const Pass &c, int idx) { return (CAUSAL && c.pass == 1) ? c.nt - 1 - idx : idx; };
+#else
+  auto tile_of = [&](const Pass &, int idx) { return idx; };
+#endif
   auto describe = [&](Pass &c) {
     c.bh = c.item / q_items;
     const int it = c.item - c.bh * q_items;
@@ -594,7 +619,11 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
     goff_v[j] = static_cast<unsigned>(row * D + (ld_pos ^ T::fv(row)) * 8) * 2u;
   }
   constexpr int kLoadsPerStep = 2 * T::kIpw;
+#ifdef KCG_FMHA_EXP_STAGE_O
+  constexpr int kStores = (OUT_BF16 ? 2 : 4) * T::kDTiles;  // vector stores of one pass's O rows
+#else
   constexpr int kStores = 4 * T::kDTiles;  // vector stores of one pass's O rows
+#endif
   constexpr int kQLoads = T::kDSteps;      // vector loads of one pass's Q rows
   const unsigned lds_k0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(Ks + ld_row0 * D));
   const unsigned lds_v0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(Vs + ld_row0 * D));
@@ -608,7 +637,7 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
   // requests the next tile of the stream; returns the number of vector memory operations issued
   auto issue_next = [&]() {
     if (!ld_valid) return 0;
-    const int kv0 = ld_tile * BC;
+    const int kv0 = tile_of(lc, ld_tile) * BC;
     const int64_t row0 = static_cast<int64_t>(lc.bh) * S + kv0;
     const char *kg = reinterpret_cast<const char *>(K + row0 * D);
     const char *vg = reinterpret_cast<const char *>(V + row0 * D);
@@ -813,6 +842,50 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
     l_run += psum;
   };
 
+#ifdef KCG_FMHA_EXP_STAGE_O
+  // normalise and store: lane holds O[wq0 + r32][32*i + 8*g + 4*half + 0..3]; 64 bytes of each
+  // of the wave's 32 rows per round go through the staging area (16-byte chunks XOR-swizzled
+  // against bank conflicts) and leave four lanes a row
+  auto store_o = [&]() {
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float inv = 1.0f / l_tot;
+    char *stage = reinterpret_cast<char *>(lds16) + T::kRingBytes + wave * T::kStageBytes;
+    char *wr = stage + r32 * 64 + 8 * half;
+    const int wswz = (r32 >> 1) & 3;
+    constexpr int kRounds = OUT_BF16 ? T::kDTiles : 2 * T::kDTiles;
+    constexpr int kRowBytes = OUT_BF16 ? 2 * D : 4 * D;
+    char *obase = static_cast<char *>(O) + (static_cast<int64_t>(cc.bh) * S + wq0) * kRowBytes;
+    const bool whole = wq0 + 32 <= S;
+#pragma unroll
+    for (int rd = 0; rd < kRounds; ++rd) {
+      if (OUT_BF16) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          u32x2_t w = {pack_bf16(acc_o[rd][4 * g + 0] * inv, acc_o[rd][4 * g + 1] * inv),
+                       pack_bf16(acc_o[rd][4 * g + 2] * inv, acc_o[rd][4 * g + 3] * inv)};
+          *reinterpret_cast<u32x2_t *>(wr + ((g ^ wswz) * 16)) = w;
+        }
+      } else {
+        // 16 columns of fp32 per round: g = 2*(rd%2) + gg, chunk = 2*gg + half
+#pragma unroll
+        for (int gg = 0; gg < 2; ++gg) {
+          const int g = 2 * (rd % 2) + gg;
+          float4_t w = {acc_o[rd / 2][4 * g + 0] * inv, acc_o[rd / 2][4 * g + 1] * inv,
+                        acc_o[rd / 2][4 * g + 2] * inv, acc_o[rd / 2][4 * g + 3] * inv};
+          *reinterpret_cast<float4_t *>(stage + r32 * 64 + (((2 * gg + half) ^ wswz) * 16)) = w;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int row = 16 * k + (lane >> 2);
+        const int chunk = lane & 3;
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + row * 64 + ((chunk ^ ((row >> 1) & 3)) * 16));
+        if (whole || wq0 + row < S)
+          *reinterpret_cast<u32x4_t *>(obase + static_cast<int64_t>(row) * kRowBytes + rd * 64 + chunk * 16) = v;
+      }
+    }
+  };
+#else
   // normalise and store: lane holds O[qrow][32*i + 8*g + 4*half + 0..3]
   auto store_o = [&]() {
     const int qrow = wq0 + r32;
@@ -838,13 +911,18 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
         }
     }
   };
+#endif
   // Stores a wave is known to issue for a pass: all of them when every row is inside the
   // sequence; a wave with rows beyond S may skip the instructions altogether, so it counts
   // none (the hand-counted waits then wait for more than they need, never for less).
   auto stores_of_pass = [&]() { return wq0 + 32 <= S ? kStores : 0; };
 
   // A wave whose last query precedes the tile has nothing to add (causal).
-  auto active = [&](int tile) { return !CAUSAL || (tile * BC <= wq0 + 31); };
+#ifdef KCG_FMHA_EXP_ALL_PAIRS
+  auto active = [&](int) { return true; };
+#else
+  auto active = [&](int idx) { return !CAUSAL || (tile_of(cc, idx) * BC <= wq0 + 31); };
+#endif
   const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   // the 2 * kDSteps MFMAs of S = K . Q^T from ring slot kslot; `primed`: the first kQueue
   // fragments are already in the queue
@@ -916,7 +994,7 @@ __global__ __launch_bounds__(512, 2) void fmha_bf16_pp_kernel(
       for (int m = 0; m < T::kQueue; ++m) oq[m] = read_v(vs_cur, m);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (act) softmax(t * BC);
+    if (act) softmax(tile_of(cc, t) * BC);
     // Still allowed in flight: the tile loads of this step and of the step before, and
     // whatever the two last matrix intervals issued after the older of them.  The K and V
     // tiles requested two steps ago are published by the coming barriers.

@@ -8,7 +8,9 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libkcg_hip.so")
+# KCG_LIBRARY names another build of the same library (the experiment builds of
+# `make -C kernelcodegen_amd/csrc variants`); unset, the library built beside this file.
+LIB_PATH = os.environ.get("KCG_LIBRARY") or os.path.join(_HERE, "libkcg_hip.so")
 
 _lib = None
 _vp = ctypes.c_void_p

@@ -170,6 +170,68 @@ def fmha(iters=20, shapes=None):
     return out
 
 
+def fmha_variants(shape=(4, 32, 4096, 128), iters=20, rounds=4):
+    """The experiment builds of the bf16 attention kernel (`make -C kernelcodegen_amd/csrc variants`)
+    against the default library on configs[4]'s shape, causal and not: every library is timed in
+    every round, one after the other, so that box and clock drift hit all of them alike; the
+    output of each build is compared with the default's (the builds change schedules, not
+    arithmetic)."""
+    import glob
+    import torch
+    from . import lib
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    paths = [lib.LIB_PATH] + sorted(glob.glob(os.path.join(here, "csrc", "variants", "libkcg_hip_*.so")))
+    if len(paths) == 1:
+        raise RuntimeError("no experiment builds: run `make -C kernelcodegen_amd/csrc variants` first")
+    libs = []
+    for p in paths:
+        L = ctypes.CDLL(p)
+        L.kcg_fmha_bf16.restype, L.kcg_fmha_bf16.argtypes = lib.SYMBOLS["kcg_fmha_bf16"]
+        libs.append(L)
+    B, H, S, D = shape
+    dev = torch.device("cuda:0")
+    _settle(dev)
+    Q = torch.randn(B, H, S, D, device=dev).to(torch.bfloat16)
+    K = torch.randn_like(Q)
+    V = torch.randn_like(Q)
+    O = torch.empty_like(Q)
+    sched = lib.FmhaSched(br=256, bc=64)
+
+    def call(L, causal):
+        lib.check(L.kcg_fmha_bf16(Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), 1, B, H, S, D,
+                                  D ** -0.5, causal, ctypes.byref(sched), lib.current_stream()))
+
+    ref = {}
+    diff = {}
+    for i, L in enumerate(libs):
+        for causal in (1, 0):
+            O.zero_()
+            call(L, causal)
+            torch.cuda.synchronize()
+            if i == 0:
+                ref[causal] = O.clone()
+            diff[(i, causal)] = float((O.float() - ref[causal].float()).abs().max())
+    best = {}
+    for _ in range(rounds):
+        for i, L in enumerate(libs):
+            for causal in (1, 0):
+                ms = _time(lambda: call(L, causal), iters)
+                best[(i, causal)] = min(ms, best.get((i, causal), ms))
+    print("shape B,H,S,D = %d,%d,%d,%d, bf16, 256-row ping-pong kernel; best of %d rounds of %d launches" % (
+        B, H, S, D, rounds, iters))
+    print("| build | causal ms | causal TFLOP/s | % of 2500 | non-causal ms | non-causal TFLOP/s | % of 2500 | max abs diff vs default |")
+    print("|---|---|---|---|---|---|---|---|")
+    for i, p in enumerate(paths):
+        name = "default" if i == 0 else os.path.basename(p)[len("libkcg_hip_"):-3]
+        fc = 2.0 * B * H * S * S * D / best[(i, 1)] / 1e9
+        fn = 4.0 * B * H * S * S * D / best[(i, 0)] / 1e9
+        print("| %s | %.4f | %.1f | %.1f | %.4f | %.1f | %.1f | %.3g / %.3g |" % (
+            name, best[(i, 1)], fc, 100 * fc / PEAK_BF16_TFLOPS, best[(i, 0)], fn, 100 * fn / PEAK_BF16_TFLOPS,
+            diff[(i, 1)], diff[(i, 0)]), flush=True)
+    return best
+
+
 def ops_chain(shape=(1, 32, 2048, 128), iters=30):
     import torch
     from . import lib, ops

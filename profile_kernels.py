@@ -35,11 +35,16 @@ def main():
     ap.add_argument("--tile", default="",
                     help="matmul workloads only: BLOCK_M x BLOCK_N x BLOCK_K of the schedule, e.g. 256x128x32 "
                          "(default: the library's choice)")
+    ap.add_argument("--library", default="",
+                    help="another build of libkcg_hip.so (an experiment build of `make -C kernelcodegen_amd/csrc "
+                         "variants`) instead of the library beside the package")
     ap.add_argument("--iters", type=int, default=200, help="launches of the workload after the settle phase")
     ap.add_argument("--settle-ms", type=float, default=40.0,
                     help="wall-clock time of the launches that precede them (0: none)")
     args = ap.parse_args()
 
+    if args.library:
+        os.environ["KCG_LIBRARY"] = os.path.abspath(args.library)
     import numpy as np
     import torch
     from kernelcodegen_amd import inputs, ops
