@@ -49,6 +49,46 @@ struct GemmDlTile {
   }
 };
 
+// ---- 96 x 96 tile on 16 x 16 x 4 MFMA blocks (gemm_f32_t96.h) ----
+// Four waves of 48 x 48 (3 x 3 blocks).  The A tile has the layout of GemmDlTile's (rows of
+// BK floats, 16-byte chunks swizzled by fa).  The B tile is stored by "row quartets": the
+// k-step s of a slice multiplies rows {4g + s : g = 0..3} of its 16-row half at once (lane
+// group g of a wave supplies row 4g + s), so those four rows are interleaved in LDS as
+// [16 columns][g][...]: quartet q = 4 * half + s holds, for every window w of 16 columns,
+// the 16 floats of row 4g + s at float offset q * 384 + w * 64 + g * 16, and a wave's
+// ds_read_b32 of one operand touches 256 consecutive bytes.
+struct GemmT96Geometry {
+  static constexpr int kBM = 96, kBN = 96, kBK = 32, kWavesM = 2, kWavesN = 2;
+  static constexpr int kWaveM = 48, kWaveN = 48, kBlocks = 3;   // 16-wide blocks per wave and side
+  static constexpr int kThreads = 256, kStages = 3;
+  static constexpr int kFloatsA = kBM * kBK, kFloatsB = kBK * kBN;
+  static constexpr int kStageFloats = kFloatsA + kFloatsB;
+  static constexpr int kLdsBytes = kStages * kStageFloats * 4;
+  static constexpr int kLoadsA = kFloatsA / 256 / 4, kLoadsB = kFloatsB / 256 / 4;  // 1 KiB loads per wave and slice
+  static constexpr int kSteps = kBK / 4;
+  static constexpr int kQuartetFloats = 4 * kBN;
+  // Chunk swizzle of the A tile (row r holds its logical 16-byte chunk c at position c ^ fa(r)).
+  // A ds_read_b128 is served in four groups of 16 lanes -- lanes {0-3, 12-15, 20-23, 24-27},
+  // {4-7, 8-11, 16-19, 28-31} and the same two sets + 32 -- and lane l reads row l % 16, chunk
+  // l / 16 of a k-half here, so a group holds all 16 rows, rows 0-3 and 12-15 with one chunk and
+  // rows 4-11 with its neighbour (chunk ^ 1).  With r / 2, flipped in its lowest bit for rows
+  // 4-11, the eight even rows of a group land in the eight 16-byte slots of one 128-byte half of
+  // the 256-byte bank window and the eight odd rows in those of the other.
+  KCG_HD static constexpr int fa(int row) {
+    const int r = row % 16;
+    return (r >> 1) ^ ((r >= 4 && r < 12) ? 1 : 0);
+  }
+  // float offset inside a slice's B tile -> (row k of the slice, first column) of that 16-byte chunk
+  KCG_HD static constexpr int b_row(int idx) {
+    const int q = idx / kQuartetFloats, in_q = idx % kQuartetFloats;
+    return 16 * (q / 4) + 4 * ((in_q % 64) / 16) + q % 4;
+  }
+  KCG_HD static constexpr int b_col(int idx) {
+    const int in_q = idx % kQuartetFloats;
+    return 16 * (in_q / 64) + in_q % 16;
+  }
+};
+
 // ---- streaming kernel (gemm_f32_stream.h) ----
 struct GemmStreamGeometry {
   static constexpr int kBM = 256, kBN = 128, kBK = 16, kWavesM = 4, kWavesN = 2;

@@ -31,6 +31,7 @@
 
 #include "gemm_dl_tile.h"
 #include "gemm_f32_stream.h"
+#include "gemm_f32_t96.h"
 #include "kcg_common.h"
 
 namespace kcg {
@@ -922,6 +923,54 @@ static GemmPlan default_plan(int64_t M, int64_t N, double *cost_out = nullptr) {
   return plan;
 }
 
+// The 96 x 96 tile (gemm_f32_t96.h): whole tiles only.
+static bool t96_shape(int64_t M, int64_t N, int64_t K) {
+  using G = GemmT96Geometry;
+  return M > 0 && N > 0 && K > 0 && M % G::kBM == 0 && N % G::kBN == 0 && K % G::kBK == 0 && K < (1 << 22) &&
+         N < (1 << 22) && (M / G::kBM) * (N / G::kBN) <= 0x7fffffffLL;
+}
+// Its cost in the units of tile_cost; negative where the tile is no candidate.  Measured
+// fraction of MFMA peak with the CUs holding R whole rounds of tiles: 0.83 (R = 1: one wave
+// per SIMD), 0.89 (2), 0.935 (4), 0.95 (9 and more), i.e. about 0.96 - 0.13 / R; scaled by
+// 0.94 like the entries of kTileCands (whose 0.91 for 256 x 128 stands for a measured 0.97).
+// Short K is left to the other tiles: this one stores C in 64-byte row segments.
+static double t96_cost(int64_t M, int64_t N, int64_t K) {
+  using G = GemmT96Geometry;
+  if (!t96_shape(M, N, K) || K < 512) return -1.0;
+  const int64_t tiles = (M / G::kBM) * (N / G::kBN);
+  if (tiles > 4096) return -1.0;
+  const double rounds = static_cast<double>((tiles + kNumCu - 1) / kNumCu);
+  return rounds * G::kBM * G::kBN / (0.94 * (0.96 - 0.13 / rounds));
+}
+// The model is good to a few per cent: the 96-wide tile must win by that much.
+constexpr double kT96Margin = 0.97;
+static int launch_t96(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
+                      int group_m, hipStream_t stream, kcg_launch_info *info) {
+  using G = GemmT96Geometry;
+  if (!t96_shape(M, N, K) || !aligned16(A) || !aligned16(B)) return KCG_ERR_BAD_SCHEDULE;
+  const int tiles_m = static_cast<int>(M / G::kBM), tiles_n = static_cast<int>(N / G::kBN);
+  if (info) {
+    *info = kcg_launch_info{};
+    info->launches = 1;
+    info->main_rows = static_cast<int>(M);
+    info->grid[0] = tiles_m * tiles_n;
+    info->grid[1] = info->grid[2] = 1;
+    info->block[0] = G::kThreads;
+    info->block[1] = info->block[2] = 1;
+    info->lds_bytes = G::kLdsBytes;
+    info->waves_per_block = G::kWavesM * G::kWavesN;
+    snprintf(info->kernel, sizeof info->kernel, "gemm_f32_96x96x32_w2x2_dl");
+    return KCG_OK;
+  }
+  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n)), block(G::kThreads);
+  auto go = [&](auto kern) {
+    if (!allow_lds(kern, G::kLdsBytes)) return static_cast<int>(KCG_ERR_LAUNCH);
+    return launch(kern, grid, block, G::kLdsBytes, stream, A, B, C, static_cast<int>(M), static_cast<int>(N),
+                  static_cast<int>(K), tiles_m, tiles_n, group_m);
+  };
+  return epilogue == KCG_EPILOGUE_RELU ? go(gemm_f32_t96_kernel<true>) : go(gemm_f32_t96_kernel<false>);
+}
+
 // Resolves a schedule (NULL / zero fields = defaults) to one of the built tile
 // shapes and either launches it or fills `info`.
 static int launch_sched(const kcg_gemm_sched &d, const float *A, const float *B, float *C, int64_t M, int64_t N,
@@ -933,6 +982,10 @@ static int launch_sched(const kcg_gemm_sched &d, const float *A, const float *B,
       d.wave_n == BN / WN)                                                                        \
     return launch_gemm<BM, BN, BK, WM, WN, MINW>(A, B, C, M, N, K, epilogue, d.group_m,           \
                                                   d.lds_stages, stream, info);
+  if (d.block_m == 96 && d.block_n == 96 && d.block_k == 32 && d.wave_m == 48 && d.wave_n == 48) {
+    if (d.lds_stages == 2) return KCG_ERR_BAD_SCHEDULE;   // built as the direct-load ring only
+    return launch_t96(A, B, C, M, N, K, epilogue, d.group_m, stream, info);
+  }
   KCG_TRY(128, 128, 32, 2, 2, 2)
   KCG_TRY(128, 128, 16, 2, 2, 2)
   KCG_TRY(128, 128, 8, 2, 2, 2)
@@ -949,11 +1002,19 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
                          kcg_launch_info *info) {
   kcg_gemm_sched d = {256, 128, 16, 8, 64, 64, 4, 64, 0};
   if (!s || (s->block_m == 0 && s->block_n == 0)) {
-    const GemmPlan plan = default_plan(M, N);
+    double plan_cost = 0.0;
+    const GemmPlan plan = default_plan(M, N, &plan_cost);
     d = plan.main;
     // a caller who fixes any tile field gets one launch with that field honoured
     const bool free_choice = !s || (s->block_k == 0 && s->wave_m == 0 && s->wave_n == 0 && s->lds_stages == 0);
     if (!free_choice) d = default_tile(M, N, 1);
+    // extents that 96 divides, where that tile fills the rounds of the CUs better
+    const double c96 = t96_cost(M, N, K);
+    if (free_choice && c96 > 0.0 && c96 < kT96Margin * plan_cost && aligned16(A) && aligned16(B) &&
+        (!s || ((s->wave_size == 0 || s->wave_size == 64) && (s->vec_width == 0 || s->vec_width == 4)))) {
+      if (s && s->group_m < 0) return KCG_ERR_BAD_SCHEDULE;
+      return launch_t96(A, B, C, M, N, K, epilogue, s && s->group_m ? s->group_m : 8, stream, info);
+    }
     if (free_choice && plan.main_rows < M) {
       // caller's remaining fields (GROUP_SIZE_M) apply to both launches
       kcg_gemm_sched t = plan.tail;
@@ -1033,6 +1094,9 @@ static bool split_tail_plan(int64_t M, int64_t N, int64_t K, int64_t max_bytes, 
   // the default plan in steps of K of a 64 x 64 tile at that tile's efficiency
   double default_area = 0.0;
   default_plan(M, N, &default_area);
+  // (the 96-wide tile competes only where it beats the split plan itself by the margin)
+  const double c96 = t96_cost(M, N, K);
+  const double plain96 = c96 > 0.0 ? c96 * small.eff / (64.0 * 64.0) * K : -1.0;
   const double plain = default_area * small.eff / (64.0 * 64.0) * K;
   const int64_t slices = K / 32;
   const int64_t max_pieces = std::min(max_bytes / kSplitPieceBytes, kSplitMaxPieces);
@@ -1056,6 +1120,7 @@ static bool split_tail_plan(int64_t M, int64_t N, int64_t K, int64_t max_bytes, 
   // bound by the host's launch rate, and two launches take twice as long as one
   // (512 x 512 x 768, 292 steps: 5 % slower; 512 x 512 x 1024, 356 steps: 30 % faster).
   if (parts == 0 || best > 0.95 * plain || plain - best < 300.0 || best < 330.0) return false;
+  if (plain96 > 0.0 && plain96 < kT96Margin * best) return false;
   out->full = static_cast<int>(rounds * kNumCu);
   out->rest = static_cast<int>(rest);
   out->parts = parts;

@@ -27,11 +27,12 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="gemm_cfg1",
                     choices=["gemm_cfg0", "gemm_cfg1", "gemm_cfg2", "fmha_cfg3", "fmha_cfg4",
-                             "bmmnt_cfg3", "bmmnn_cfg3", "softmax_cfg3", "relu_1gib", "gemm_ksplit"],
+                             "bmmnt_cfg3", "bmmnn_cfg3", "softmax_cfg3", "relu_1gib", "gemm_ksplit", "gemm_1536"],
                     help="a BASELINE config of the fused kernels, or an un-fused operator at the "
                          "configs[3] shape (bmmnt: Q.K^T, bmmnn: P.V, softmax: in place on the scores) "
                          "/ ReLU on a 1 GiB tensor / gemm_ksplit: 1536^3 (+ReLU) through the workspace entry "
-                         "point, whose plan is two launches (whole tiles and K pieces, then the sum of the pieces)")
+                         "point, whose plan is two launches (whole tiles and K pieces, then the sum of the pieces) "
+                         "/ gemm_1536: 1536^3 (+ReLU) through kcg_gemm_f32 (the 96 x 96 tile by default; --tile applies)")
     ap.add_argument("--tile", default="",
                     help="matmul workloads only: BLOCK_M x BLOCK_N x BLOCK_K of the schedule, e.g. 256x128x32 "
                          "(default: the library's choice)")
@@ -82,6 +83,16 @@ def main():
         ws = torch.empty(ops.matmul_workspace_bytes(d, d, d) // 4, dtype=torch.float32, device=dev)
         assert ws.numel() > 0
         fn = lambda: ops.matmul(A, B, relu=True, out=C, workspace=ws)
+    elif args.workload == "gemm_1536":
+        d = 1536
+        A = torch.empty(d, d, device=dev).normal_()
+        B = torch.empty(d, d, device=dev).normal_()
+        C = torch.empty(d, d, device=dev)
+        sched = None
+        if args.tile:
+            bm, bn, bk = (int(x) for x in args.tile.split("x"))
+            sched = dict(block_m=bm, block_n=bn, block_k=bk)
+        fn = lambda: ops.matmul(A, B, relu=True, out=C, sched=sched)
     elif kind == "gemm":
         A = torch.from_numpy(c["A"]).to(dev)
         B = torch.from_numpy(c["B"]).to(dev)

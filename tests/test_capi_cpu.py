@@ -88,6 +88,26 @@ def test_launch_geometry_queries():
     s = lib.GemmSched(block_m=256, block_n=128, block_k=16, wave_m=64, wave_n=64)
     assert L.kcg_gemm_f32_query(7168, 7168, 7168, ctypes.byref(s), ctypes.byref(info)) == 0
     assert info.grid[0] == 28 * 56 and b"+" not in info.kernel
+    # 1536^3: 576 tiles of 64 x 64 are 2.25 rounds of the 256 CUs, 256 tiles of 96 x 96 exactly one
+    assert L.kcg_gemm_f32_query(1536, 1536, 1536, None, ctypes.byref(info)) == 0
+    assert info.kernel == b"gemm_f32_96x96x32_w2x2_dl" and info.launches == 1
+    assert info.grid[0] == 256 and info.block[0] == 256 and info.waves_per_block == 4
+    assert info.lds_bytes == 3 * (96 * 32 + 32 * 96) * 4
+    # ... also when only GROUP_SIZE_M is given; with a short K the power-of-two tiles keep the problem
+    assert L.kcg_gemm_f32_query(1536, 1536, 1536, ctypes.byref(lib.GemmSched(group_m=4)), ctypes.byref(info)) == 0
+    assert info.kernel == b"gemm_f32_96x96x32_w2x2_dl"
+    assert L.kcg_gemm_f32_query(1536, 1536, 256, None, ctypes.byref(info)) == 0
+    assert b"96x96" not in info.kernel
+    # the tile by name: whole tiles only, direct-load ring only
+    s96 = lib.GemmSched(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
+    assert L.kcg_gemm_f32_query(960, 192, 64, ctypes.byref(s96), ctypes.byref(info)) == 0
+    assert info.grid[0] == 10 * 2 and info.kernel == b"gemm_f32_96x96x32_w2x2_dl"
+    assert L.kcg_gemm_f32_query(960, 200, 64, ctypes.byref(s96), ctypes.byref(info)) == 4
+    assert L.kcg_gemm_f32_query(960, 192, 48, ctypes.byref(s96), ctypes.byref(info)) == 4
+    s96.lds_stages = 2
+    assert L.kcg_gemm_f32_query(960, 192, 64, ctypes.byref(s96), ctypes.byref(info)) == 4
+    s96.lds_stages, s96.wave_m = 3, 32
+    assert L.kcg_gemm_f32_query(960, 192, 64, ctypes.byref(s96), ctypes.byref(info)) == 4
     # bf16 causal, S = 4096: 256-row query blocks run in pairs (n-1-i, i) -> 8 work items per
     # head, 1024 in all, walked by one persistent 8-wave workgroup per CU
     assert L.kcg_fmha_query(1, 4, 32, 4096, 128, 1, None, ctypes.byref(info)) == 0

@@ -124,3 +124,29 @@ def test_k_split_launch_numbering_and_addresses(model, shape):
                            capture_output=True, text=True, timeout=300)
         assert r.returncode == 0, r.stdout + r.stderr
         assert " 0 violations" in r.stdout
+
+
+# ---- the 96 x 96 tile on 16 x 16 x 4 MFMA blocks (gemm_f32_t96_kernel) ----
+T96_SRC = os.path.join(ROOT, "tests", "gemm_t96_address_model.cc")
+
+
+@pytest.fixture(scope="module")
+def t96_model(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("gemm_t96") / "gemm_t96_address_model")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-I", INC, T96_SRC, "-o", exe], check=True)
+    return exe
+
+
+# (M, N, K, GROUP_M): one tile and one slice, the size the tile exists for, tile counts the
+# XCD count and GROUP_M do not divide, lane offsets close to 2^32 / byte offsets beyond it
+@pytest.mark.parametrize("case", [(96, 96, 32, 8), (1536, 1536, 1536, 8), (960, 4128, 64, 3), (672, 1248, 4000 // 32 * 32, 5),
+                                  (40032, 384, 32768, 8), (192, 3999936, 32, 8)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_t96_loads_operands_and_stores(t96_model, case):
+    """The direct loads of a slice fill its A and B stage exactly once from inside the
+    tensors; every operand read of every lane fetches the (row, k) / (k, column) its MFMA step
+    multiplies, both operands with the same k and every k of the slice once; the stores of
+    the four waves cover the C tile exactly once."""
+    r = subprocess.run([t96_model] + [str(v) for v in case], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert " 0 violations" in r.stdout

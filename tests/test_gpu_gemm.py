@@ -146,6 +146,68 @@ def test_relu_epilogue_special_values(dev):
     assert C[4, 9] == 0 and C[5, 10] == np.inf and np.isnan(C[6, 11])
 
 
+T96 = dict(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
+
+
+# K of 1, 2, 3, 5, 48 and 124 slices: every phase of the three-stage ring (K / 32 mod 3 = 1, 2, 0)
+@pytest.mark.parametrize("shape", [(96, 96, 32), (96, 192, 64), (288, 96, 96), (480, 672, 160), (1536, 1536, 1536),
+                                   (960, 1152, 3968)])
+def test_tile_96(oracle, dev, shape):
+    """The 96 x 96 x 32 tile (four waves of 48 x 48 on 16 x 16 x 4 MFMA blocks) by name."""
+    from kernelcodegen_amd import ops
+    M, N, K = shape
+    A = inputs.uniform((M, K), 111, 0)
+    B = inputs.uniform((K, N), 111, 1)
+    ref = oracle.matmul(A, B)
+    C = ops.matmul(_gpu(A, dev), _gpu(B, dev), sched=T96).cpu().numpy()
+    assert max(rel_err(C, ref)) < TOL
+    Cr = ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=True, sched=T96).cpu().numpy()
+    assert np.array_equal(Cr, oracle.relu(C))
+    assert max(rel_err(Cr, oracle.relu(ref))) < TOL
+
+
+def test_tile_96_closed_forms_and_default_choice(dev):
+    import torch
+    from kernelcodegen_amd import ops, lib
+    from kernelcodegen_amd.lib import KcgError
+    rng = np.random.default_rng(5)
+    # small integers: exact in fp32 whatever the summation order
+    Ai = rng.integers(-8, 9, (288, 512)).astype(np.float32)
+    Bi = rng.integers(-8, 9, (512, 384)).astype(np.float32)
+    expect = (Ai.astype(np.int64) @ Bi.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(ops.matmul(_gpu(Ai, dev), _gpu(Bi, dev), sched=T96).cpu().numpy(), expect)
+    # lane mapping of rows, columns and k: A[i,k] = i with B = e_k0 (row k0 of ones) gives C[i,j] = i
+    # for every k0 of a slice; A = ones with B[k,j] = j * [k == k0] gives C[i,j] = j
+    Am = np.repeat(np.arange(192, dtype=np.float32)[:, None], 64, axis=1)
+    for k0 in (0, 5, 19, 31, 32 + 14, 63):
+        Bm = np.zeros((64, 288), np.float32)
+        Bm[k0] = 1
+        got = ops.matmul(_gpu(Am, dev), _gpu(Bm, dev), sched=T96).cpu().numpy()
+        assert np.array_equal(got, np.repeat(np.arange(192, dtype=np.float32)[:, None], 288, axis=1)), k0
+        Bj = np.zeros((64, 288), np.float32)
+        Bj[k0] = np.arange(288)
+        Ak = np.zeros((192, 64), np.float32)
+        Ak[:, k0] = 1          # only k0 may be picked up: any other k of A against row k0 of B is 0
+        got = ops.matmul(_gpu(Ak, dev), _gpu(Bj, dev), sched=T96).cpu().numpy()
+        assert np.array_equal(got, np.repeat(np.arange(288, dtype=np.float32)[None, :], 192, axis=0)), k0
+    # 1536^3 takes this tile by default (256 tiles on 256 CUs); GROUP_SIZE_M only renumbers them
+    info = lib.LaunchInfo()
+    import ctypes
+    assert lib.load().kcg_gemm_f32_query(1536, 1536, 1536, None, ctypes.byref(info)) == 0
+    assert info.kernel == b"gemm_f32_96x96x32_w2x2_dl"
+    A = torch.randn(1536, 1536, device=dev)
+    B = torch.randn(1536, 1536, device=dev)
+    base = ops.matmul(A, B, relu=True)
+    assert torch.equal(base, ops.matmul(A, B, relu=True, sched=T96))
+    for g in (1, 3, 5):
+        assert torch.equal(base, ops.matmul(A, B, relu=True, sched=dict(group_m=g)))
+    # whole tiles only
+    with pytest.raises(KcgError):
+        ops.matmul(torch.randn(100, 64, device=dev), torch.randn(64, 96, device=dev), sched=T96)
+    with pytest.raises(KcgError):
+        ops.matmul(torch.randn(96, 48, device=dev), torch.randn(48, 96, device=dev), sched=T96)
+
+
 def test_row_permutation_is_bit_exact(dev):
     import torch
     from kernelcodegen_amd import ops

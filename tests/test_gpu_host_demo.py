@@ -164,13 +164,29 @@ def test_matmul_config_search(oracle, dev, tmp_path):
     got, text = _run(["tune", "matmul", M, N, K, 1], tmp_path)
     trials, best = _trials(text)
     assert [t[0] for t in trials] == ["256x128x16", "256x128x32", "128x128x16", "128x128x32", "128x128x8",
-                                      "128x64x32", "64x64x32"]
+                                      "128x64x32", "64x64x32", "96x96x32"]
     timed = [t for t in trials if t[2] is not None]
-    assert len(timed) == 7 and all(0 < t[2] < 50 for t in timed)
+    # (96 does not divide 2048: that tile takes whole tiles only and is refused)
+    assert len(timed) == 7 and all(0 < t[2] < 50 for t in timed) and trials[-1][2] is None
     fastest = min(timed, key=lambda t: t[2])
     assert best is not None and best[0] == fastest[0] and abs(best[1] - fastest[2]) < 1e-4
     bm, bn, bk = (int(x) for x in best[0].split("x"))
     assert "static const kcg_gemm_sched sched = {%d, %d, %d," % (bm, bn, bk) in text
+    A = inputs.uniform((M, K), SEED, 0)
+    B = inputs.uniform((K, N), SEED, 1)
+    ref = oracle.relu(oracle.matmul(A, B))
+    assert max(rel_err(got.reshape(M, N), ref)) < 1e-4
+
+
+def test_matmul_config_search_finds_the_96_tile(oracle, dev, tmp_path):
+    """1536^3: 256 tiles of 96 x 96 are exactly one round of the CUs, every power-of-two tile
+    leaves a partly filled one; the measured search picks it."""
+    M = N = K = 1536
+    got, text = _run(["tune", "matmul", M, N, K, 1], tmp_path)
+    trials, best = _trials(text)
+    assert all(t[2] is not None for t in trials) and len(trials) == 8
+    assert best is not None and best[0] == "96x96x32"
+    assert "static const kcg_gemm_sched sched = {96, 96, 32," in text
     A = inputs.uniform((M, K), SEED, 0)
     B = inputs.uniform((K, N), SEED, 1)
     ref = oracle.relu(oracle.matmul(A, B))
