@@ -923,11 +923,11 @@ static GemmPlan default_plan(int64_t M, int64_t N, double *cost_out = nullptr) {
   return plan;
 }
 
-// The 96 x 96 tile (gemm_f32_t96.h): whole tiles only.
+// The 96 x 96 tile (gemm_f32_t96.h): K in whole slices, rows 16-byte aligned.
 static bool t96_shape(int64_t M, int64_t N, int64_t K) {
   using G = GemmT96Geometry;
-  return M > 0 && N > 0 && K > 0 && M % G::kBM == 0 && N % G::kBN == 0 && K % G::kBK == 0 && K < (1 << 22) &&
-         N < (1 << 22) && (M / G::kBM) * (N / G::kBN) <= 0x7fffffffLL;
+  return M > 0 && N > 0 && K > 0 && N % 4 == 0 && K % G::kBK == 0 && K < (1 << 22) && N < (1 << 22) &&
+         M <= 0x7fffffffLL && ((M + G::kBM - 1) / G::kBM) * ((N + G::kBN - 1) / G::kBN) <= 0x7fffffffLL;
 }
 // Its cost in the units of tile_cost; negative where the tile is no candidate.  Measured
 // fraction of MFMA peak with the CUs holding R whole rounds of tiles: 0.83 (R = 1: one wave
@@ -937,7 +937,7 @@ static bool t96_shape(int64_t M, int64_t N, int64_t K) {
 static double t96_cost(int64_t M, int64_t N, int64_t K) {
   using G = GemmT96Geometry;
   if (!t96_shape(M, N, K) || K < 512) return -1.0;
-  const int64_t tiles = (M / G::kBM) * (N / G::kBN);
+  const int64_t tiles = ((M + G::kBM - 1) / G::kBM) * ((N + G::kBN - 1) / G::kBN);
   if (tiles > 4096) return -1.0;
   const double rounds = static_cast<double>((tiles + kNumCu - 1) / kNumCu);
   return rounds * G::kBM * G::kBN / (0.94 * (0.96 - 0.13 / rounds));
@@ -948,7 +948,8 @@ static int launch_t96(const float *A, const float *B, float *C, int64_t M, int64
                       int group_m, hipStream_t stream, kcg_launch_info *info) {
   using G = GemmT96Geometry;
   if (!t96_shape(M, N, K) || !aligned16(A) || !aligned16(B)) return KCG_ERR_BAD_SCHEDULE;
-  const int tiles_m = static_cast<int>(M / G::kBM), tiles_n = static_cast<int>(N / G::kBN);
+  const int tiles_m = static_cast<int>((M + G::kBM - 1) / G::kBM), tiles_n = static_cast<int>((N + G::kBN - 1) / G::kBN);
+  const bool ragged = M % G::kBM != 0 || N % G::kBN != 0;
   if (info) {
     *info = kcg_launch_info{};
     info->launches = 1;
@@ -959,7 +960,7 @@ static int launch_t96(const float *A, const float *B, float *C, int64_t M, int64
     info->block[1] = info->block[2] = 1;
     info->lds_bytes = G::kLdsBytes;
     info->waves_per_block = G::kWavesM * G::kWavesN;
-    snprintf(info->kernel, sizeof info->kernel, "gemm_f32_96x96x32_w2x2_dl");
+    snprintf(info->kernel, sizeof info->kernel, "gemm_f32_96x96x32_w2x2_dl%s", ragged ? "_ragged" : "");
     return KCG_OK;
   }
   const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n)), block(G::kThreads);
@@ -968,7 +969,9 @@ static int launch_t96(const float *A, const float *B, float *C, int64_t M, int64
     return launch(kern, grid, block, G::kLdsBytes, stream, A, B, C, static_cast<int>(M), static_cast<int>(N),
                   static_cast<int>(K), tiles_m, tiles_n, group_m);
   };
-  return epilogue == KCG_EPILOGUE_RELU ? go(gemm_f32_t96_kernel<true>) : go(gemm_f32_t96_kernel<false>);
+  const bool relu = epilogue == KCG_EPILOGUE_RELU;
+  if (ragged) return relu ? go(gemm_f32_t96_kernel<true, true>) : go(gemm_f32_t96_kernel<false, true>);
+  return relu ? go(gemm_f32_t96_kernel<true, false>) : go(gemm_f32_t96_kernel<false, false>);
 }
 
 // Resolves a schedule (NULL / zero fields = defaults) to one of the built tile

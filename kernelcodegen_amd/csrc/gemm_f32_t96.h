@@ -1,6 +1,6 @@
-// fp32 matmul on a 96 x 96 tile: the tile for problems whose extents 96 divides and whose
-// tile count then fills the 256 CUs in whole rounds where the power-of-two tiles do not
-// (1536^3 is 256 tiles of 96 x 96, but 576 = 2.25 x 256 tiles of 64 x 64).
+// fp32 matmul on a 96 x 96 tile: the tile for problems whose count of such tiles fills the
+// 256 CUs in whole rounds where the power-of-two tiles do not (1536^3 is 256 tiles of
+// 96 x 96, but 576 = 2.25 x 256 tiles of 64 x 64).
 //
 // Same schedule as gemm_f32_dl_kernel (MatmulOptimizer's, src/Optimizer/Optimizer.cc:383-548:
 // a tile of C per workgroup, K in BLOCK_SIZE_K slices through a ring of LDS stages, later
@@ -13,7 +13,10 @@
 // slice; the j-th MFMA of that half consumes k = 4g + j from both operands, so the products
 // summed into an element of C are those of the reference nest in a different order.
 //
-// Whole tiles only: M and N multiples of 96, K a multiple of 32, rows 16-byte aligned.
+// K is a multiple of 32 and N of 4 (rows keep 16-byte alignment).  RAGGED: M and N need not
+// divide the tile.  Rows of A at and beyond M and 16-byte column chunks of B at and beyond N
+// only feed elements of C that are never stored, so their lanes fetch the last valid row /
+// chunk instead (a loop-invariant change of the lane offsets), and the stores are bounds-checked.
 #pragma once
 
 #include <type_traits>
@@ -23,13 +26,12 @@
 
 namespace kcg {
 
-template <bool RELU>
+template <bool RELU, bool RAGGED>
 __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N, int K,
     int tiles_m, int tiles_n, int group_m) {
   using G = GemmT96Geometry;
   extern __shared__ __align__(16) float lds[];
-  (void)M;
 
   const int logical = xcd_contiguous_id(blockIdx.x, tiles_m * tiles_n);
   const int width = group_m * tiles_n;
@@ -63,12 +65,15 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
     const int idx = (wave * G::kLoadsA + i) * 256 + lane * 4;  // float index in the LDS A tile
     const int row = idx / G::kBK;
     const int c_log = ((idx % G::kBK) / 4) ^ G::fa(row);
-    oa[i] = static_cast<unsigned>(row * K + 4 * c_log) * 4u;
+    const int grow = RAGGED ? (row < M - m0 ? row : M - m0 - 1) : row;
+    oa[i] = static_cast<unsigned>(grow * K + 4 * c_log) * 4u;
   }
 #pragma unroll
   for (int i = 0; i < G::kLoadsB; ++i) {
     const int idx = (wave * G::kLoadsB + i) * 256 + lane * 4;  // float index in the LDS B tile
-    ob[i] = static_cast<unsigned>(G::b_row(idx) * N + G::b_col(idx)) * 4u;
+    const int col = G::b_col(idx);
+    const int gcol = RAGGED ? (col < N - n0 ? col : N - n0 - 4) : col;
+    ob[i] = static_cast<unsigned>(G::b_row(idx) * N + gcol) * 4u;
   }
   const char *ga = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
   const char *gb = reinterpret_cast<const char *>(B + n0);
@@ -222,7 +227,8 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
 
   // 16 lanes write 64 consecutive bytes of a row of C
-  float *c_lane = C + static_cast<int64_t>(m0 + wm * G::kWaveM + 4 * g) * N + (n0 + wn * G::kWaveN + r16);
+  const int row0 = m0 + wm * G::kWaveM + 4 * g, col0 = n0 + wn * G::kWaveN + r16;
+  float *c_lane = C + static_cast<int64_t>(row0) * N + col0;
 #pragma unroll
   for (int i = 0; i < G::kBlocks; ++i)
 #pragma unroll
@@ -231,7 +237,8 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
       for (int e = 0; e < 4; ++e) {
         float v = acc[i][n][e];
         if (RELU) v = relu_maxf(v);
-        c_lane[static_cast<int64_t>(i * 16 + e) * N + n * 16] = v;
+        if (!RAGGED || (row0 + i * 16 + e < M && col0 + n * 16 < N))
+          c_lane[static_cast<int64_t>(i * 16 + e) * N + n * 16] = v;
       }
 }
 

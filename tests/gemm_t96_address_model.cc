@@ -6,7 +6,8 @@
 //   * the element an operand read fetches from the filled stage is the one the MFMA step
 //     multiplies: A[m0 + row][k] and B[k][n0 + col] with the same k for both operands, each k
 //     of the slice exactly once per (row, col);
-//   * the stores cover the C tile exactly once, inside C.
+//   * the stores cover the part of the C tile that lies inside C exactly once (M and N need
+//     not divide the tile: lanes beyond an edge load the last valid row / chunk).
 // usage: gemm_t96_address_model M N K GROUP_M   (prints "... N violations")
 #include <cstdint>
 #include <cstdio>
@@ -32,8 +33,8 @@ int main(int argc, char **argv) {
   if (argc != 5) return 2;
   const int64_t M = atoll(argv[1]), N = atoll(argv[2]), K = atoll(argv[3]);
   const int group_m = atoi(argv[4]);
-  if (M % G::kBM || N % G::kBN || K % G::kBK) return 2;
-  const int tiles_m = static_cast<int>(M / G::kBM), tiles_n = static_cast<int>(N / G::kBN);
+  if (N % 4 || K % G::kBK) return 2;
+  const int tiles_m = static_cast<int>((M + G::kBM - 1) / G::kBM), tiles_n = static_cast<int>((N + G::kBN - 1) / G::kBN);
   const int grid = tiles_m * tiles_n;
   const int64_t a_bytes = M * K * 4, b_bytes = K * N * 4, c_elems = M * N;
   std::vector<int> seen_tile(grid, 0);
@@ -63,7 +64,9 @@ int main(int argc, char **argv) {
           const int idx = (wave * G::kLoadsA + i) * 256 + lane * 4;
           const int row = idx / G::kBK;
           const int c_log = ((idx % G::kBK) / 4) ^ G::fa(row);
-          const uint64_t off64 = (static_cast<uint64_t>(row) * K + 4 * c_log) * 4u;
+          // (rows at and beyond M: the last valid row instead)
+          const int64_t grow = row < M - m0 ? row : M - m0 - 1;
+          const uint64_t off64 = (static_cast<uint64_t>(grow) * K + 4 * c_log) * 4u;
           if (off64 > 0xffffffffull) fail("A lane offset overflows 32 bits", row, c_log, 0);
           for (int64_t kt = 0; kt < K / G::kBK; kt += (K / G::kBK > 2 ? K / G::kBK - 1 : 1)) {
             const int64_t byte = (m0 * K + kt * G::kBK) * 4 + static_cast<int64_t>(off64);
@@ -77,8 +80,11 @@ int main(int argc, char **argv) {
         for (int i = 0; i < G::kLoadsB; ++i) {
           const int idx = (wave * G::kLoadsB + i) * 256 + lane * 4;
           const int row = G::b_row(idx), col = G::b_col(idx);
-          const uint64_t off64 = (static_cast<uint64_t>(row) * N + col) * 4u;
+          // (column chunks at and beyond N: the last valid chunk instead)
+          const int64_t gcol = col < N - n0 ? col : N - n0 - 4;
+          const uint64_t off64 = (static_cast<uint64_t>(row) * N + gcol) * 4u;
           if (off64 > 0xffffffffull) fail("B lane offset overflows 32 bits", row, col, 0);
+          if (gcol < 0) fail("B chunk clamped below the tile", block, col, 0);
           if (row < 0 || row >= G::kBK || col < 0 || col + 4 > G::kBN) fail("B chunk outside the slice", idx, row, col);
           for (int64_t kt = 0; kt < K / G::kBK; kt += (K / G::kBK > 2 ? K / G::kBK - 1 : 1)) {
             const int64_t byte = (kt * G::kBK * N + n0) * 4 + static_cast<int64_t>(off64);
@@ -122,6 +128,7 @@ int main(int argc, char **argv) {
           for (int n = 0; n < G::kBlocks; ++n)
             for (int e = 0; e < 4; ++e) {
               const int row = wm * G::kWaveM + i * 16 + 4 * g + e, col = wn * G::kWaveN + n * 16 + r16;
+              if (m0 + row >= M || n0 + col >= N) continue;   // the kernel's bounds check
               ++c_cover[row * G::kBN + col];
               const int64_t elem = (m0 + row) * N + n0 + col;
               if (elem < 0 || elem >= c_elems) fail("store outside C", block, row, col);
@@ -137,8 +144,10 @@ int main(int argc, char **argv) {
         kmask |= bit;
       }
     if (kmask != 0xffffffffu) fail("the steps of a slice do not cover its 32 k", kmask, 0, 0);
-    for (int v : c_cover)
-      if (v != 1) fail("C element stored other than once", v, 0, 0);
+    for (int row = 0; row < G::kBM; ++row)
+      for (int col = 0; col < G::kBN; ++col)
+        if (c_cover[row * G::kBN + col] != ((m0 + row < M && n0 + col < N) ? 1 : 0))
+          fail("C element of the tile stored other than once / outside C", block, row, col);
   }
   for (int t = 0; t < grid; ++t)
     if (seen_tile[t] != 1) fail("tile computed other than once", t, seen_tile[t], 0);

@@ -98,11 +98,16 @@ def test_launch_geometry_queries():
     assert info.kernel == b"gemm_f32_96x96x32_w2x2_dl"
     assert L.kcg_gemm_f32_query(1536, 1536, 256, None, ctypes.byref(info)) == 0
     assert b"96x96" not in info.kernel
-    # the tile by name: whole tiles only, direct-load ring only
+    # 1472^3: 16 x 16 tiles of 96 x 96 (the last ones partly outside C) are one round as well
+    assert L.kcg_gemm_f32_query(1472, 1472, 1472, None, ctypes.byref(info)) == 0
+    assert info.kernel == b"gemm_f32_96x96x32_w2x2_dl_ragged" and info.grid[0] == 256
+    # the tile by name: K in whole slices, N a multiple of 4, direct-load ring only
     s96 = lib.GemmSched(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
     assert L.kcg_gemm_f32_query(960, 192, 64, ctypes.byref(s96), ctypes.byref(info)) == 0
     assert info.grid[0] == 10 * 2 and info.kernel == b"gemm_f32_96x96x32_w2x2_dl"
-    assert L.kcg_gemm_f32_query(960, 200, 64, ctypes.byref(s96), ctypes.byref(info)) == 4
+    assert L.kcg_gemm_f32_query(950, 200, 64, ctypes.byref(s96), ctypes.byref(info)) == 0
+    assert info.grid[0] == 10 * 3 and info.kernel == b"gemm_f32_96x96x32_w2x2_dl_ragged"
+    assert L.kcg_gemm_f32_query(960, 198, 64, ctypes.byref(s96), ctypes.byref(info)) == 4
     assert L.kcg_gemm_f32_query(960, 192, 48, ctypes.byref(s96), ctypes.byref(info)) == 4
     s96.lds_stages = 2
     assert L.kcg_gemm_f32_query(960, 192, 64, ctypes.byref(s96), ctypes.byref(info)) == 4

@@ -138,15 +138,17 @@ def t96_model(tmp_path_factory):
 
 
 # (M, N, K, GROUP_M): one tile and one slice, the size the tile exists for, tile counts the
-# XCD count and GROUP_M do not divide, lane offsets close to 2^32 / byte offsets beyond it
+# XCD count and GROUP_M do not divide, lane offsets close to 2^32 / byte offsets beyond it,
+# and extents 96 does not divide (a single row, a single column chunk, edges in M, N and both)
 @pytest.mark.parametrize("case", [(96, 96, 32, 8), (1536, 1536, 1536, 8), (960, 4128, 64, 3), (672, 1248, 4000 // 32 * 32, 5),
-                                  (40032, 384, 32768, 8), (192, 3999936, 32, 8)],
+                                  (40032, 384, 32768, 8), (192, 3999936, 32, 8), (1, 4, 32, 8), (97, 100, 96, 3),
+                                  (1472, 1500, 64, 8), (40000, 388, 32768, 8)],
                          ids=lambda c: "x".join(map(str, c)))
 def test_t96_loads_operands_and_stores(t96_model, case):
     """The direct loads of a slice fill its A and B stage exactly once from inside the
     tensors; every operand read of every lane fetches the (row, k) / (k, column) its MFMA step
     multiplies, both operands with the same k and every k of the slice once; the stores of
-    the four waves cover the C tile exactly once."""
+    the four waves cover the part of the C tile inside C exactly once."""
     r = subprocess.run([t96_model] + [str(v) for v in case], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stdout + r.stderr
     assert " 0 violations" in r.stdout

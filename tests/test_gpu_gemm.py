@@ -150,8 +150,10 @@ T96 = dict(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
 
 
 # K of 1, 2, 3, 5, 48 and 124 slices: every phase of the three-stage ring (K / 32 mod 3 = 1, 2, 0)
+# and extents 96 does not divide: one row, one column chunk, edges in M, in N and in both
 @pytest.mark.parametrize("shape", [(96, 96, 32), (96, 192, 64), (288, 96, 96), (480, 672, 160), (1536, 1536, 1536),
-                                   (960, 1152, 3968)])
+                                   (960, 1152, 3968), (1, 4, 32), (97, 100, 96), (200, 96, 64), (192, 260, 128),
+                                   (1472, 1472, 1472), (1000, 1500, 544)])
 def test_tile_96(oracle, dev, shape):
     """The 96 x 96 x 32 tile (four waves of 48 x 48 on 16 x 16 x 4 MFMA blocks) by name."""
     from kernelcodegen_amd import ops
@@ -201,9 +203,17 @@ def test_tile_96_closed_forms_and_default_choice(dev):
     assert torch.equal(base, ops.matmul(A, B, relu=True, sched=T96))
     for g in (1, 3, 5):
         assert torch.equal(base, ops.matmul(A, B, relu=True, sched=dict(group_m=g)))
-    # whole tiles only
+    # ragged output is not touched outside C
+    M, N, K = 190, 100, 64
+    buf = torch.full((1000 + M * N + 1000,), 7.0, device=dev)
+    Cv = buf[1000:1000 + M * N].view(M, N)
+    Ar, Br = torch.randn(M, K, device=dev), torch.randn(K, N, device=dev)
+    ops.matmul(Ar, Br, out=Cv, sched=T96)
+    assert bool((buf[:1000] == 7.0).all()) and bool((buf[1000 + M * N:] == 7.0).all())
+    assert torch.allclose(Cv, Ar @ Br, rtol=1e-4, atol=1e-3)
+    # K in whole slices and N a multiple of 4 only
     with pytest.raises(KcgError):
-        ops.matmul(torch.randn(100, 64, device=dev), torch.randn(64, 96, device=dev), sched=T96)
+        ops.matmul(torch.randn(100, 64, device=dev), torch.randn(64, 98, device=dev), sched=T96)
     with pytest.raises(KcgError):
         ops.matmul(torch.randn(96, 48, device=dev), torch.randn(48, 96, device=dev), sched=T96)
 
