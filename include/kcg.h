@@ -71,8 +71,8 @@ typedef enum kcg_epilogue { KCG_EPILOGUE_NONE = 0, KCG_EPILOGUE_RELU = 1 } kcg_e
  * wave64, 64 x 64 per-wave tile of 32x32x2 fp32 MFMA blocks, group_m 8; with no tile
  * given the library picks among its tiles by problem size).  Built tiles (block_m x
  * block_n x block_k, wave_m x wave_n): 256x128x{16,32} and 128x128x{8,16,32} in waves of
- * 64x64, 128x64x32 in 64x32, 64x64x32 in 32x32, and 96x96x32 in waves of 48x48 (16x16x4
- * MFMA blocks; K a multiple of 32 and N of 4, else KCG_ERR_BAD_SCHEDULE). */
+ * 64x64, 128x64x32 in 64x32, 64x64x32 in 32x32, and 96x96x32 / 96x64x32 in waves of 48x48 /
+ * 48x32 (16x16x4 MFMA blocks; K a multiple of 32 and N of 4, else KCG_ERR_BAD_SCHEDULE). */
 typedef struct kcg_gemm_sched {
   int32_t block_m;   /* BLOCK_SIZE_M: rows of C per workgroup                  */
   int32_t block_n;   /* BLOCK_SIZE_N: columns of C per workgroup               */

@@ -49,17 +49,19 @@ struct GemmDlTile {
   }
 };
 
-// ---- 96 x 96 tile on 16 x 16 x 4 MFMA blocks (gemm_f32_t96.h) ----
-// Four waves of 48 x 48 (3 x 3 blocks).  The A tile has the layout of GemmDlTile's (rows of
-// BK floats, 16-byte chunks swizzled by fa).  The B tile is stored by "row quartets": the
-// k-step s of a slice multiplies rows {4g + s : g = 0..3} of its 16-row half at once (lane
-// group g of a wave supplies row 4g + s), so those four rows are interleaved in LDS as
-// [16 columns][g][...]: quartet q = 4 * half + s holds, for every window w of 16 columns,
-// the 16 floats of row 4g + s at float offset q * 384 + w * 64 + g * 16, and a wave's
+// ---- tiles on 16 x 16 x 4 MFMA blocks: 96 x 96 and 96 x 64 (gemm_f32_t96.h) ----
+// Four waves (2 x 2) of BM/2 x BN/2, i.e. BM/32 x BN/32 blocks each; K slices of 32.  The A
+// tile has rows of 32 floats with their 16-byte chunks swizzled by fa.  The B tile is stored
+// by "row quartets": the k-step s of a slice multiplies rows {4g + s : g = 0..3} of its
+// 16-row half at once (lane group g of a wave supplies row 4g + s), so those four rows are
+// interleaved in LDS: quartet q = 4 * half + s holds, for every window w of 16 columns, the
+// 16 floats of row 4g + s at float offset q * 4 * BN + w * 64 + g * 16, and a wave's
 // ds_read_b32 of one operand touches 256 consecutive bytes.
-struct GemmT96Geometry {
-  static constexpr int kBM = 96, kBN = 96, kBK = 32, kWavesM = 2, kWavesN = 2;
-  static constexpr int kWaveM = 48, kWaveN = 48, kBlocks = 3;   // 16-wide blocks per wave and side
+template <int BM, int BN>
+struct GemmT96Tile {
+  static constexpr int kBM = BM, kBN = BN, kBK = 32, kWavesM = 2, kWavesN = 2;
+  static constexpr int kWaveM = BM / 2, kWaveN = BN / 2;
+  static constexpr int kBlocksM = kWaveM / 16, kBlocksN = kWaveN / 16;   // 16-wide blocks per wave
   static constexpr int kThreads = 256, kStages = 3;
   static constexpr int kFloatsA = kBM * kBK, kFloatsB = kBK * kBN;
   static constexpr int kStageFloats = kFloatsA + kFloatsB;
@@ -67,6 +69,7 @@ struct GemmT96Geometry {
   static constexpr int kLoadsA = kFloatsA / 256 / 4, kLoadsB = kFloatsB / 256 / 4;  // 1 KiB loads per wave and slice
   static constexpr int kSteps = kBK / 4;
   static constexpr int kQuartetFloats = 4 * kBN;
+  static_assert(BM % 32 == 0 && BN % 32 == 0, "whole 1 KiB loads per wave, whole blocks per wave");
   // Chunk swizzle of the A tile (row r holds its logical 16-byte chunk c at position c ^ fa(r)).
   // A ds_read_b128 is served in four groups of 16 lanes -- lanes {0-3, 12-15, 20-23, 24-27},
   // {4-7, 8-11, 16-19, 28-31} and the same two sets + 32 -- and lane l reads row l % 16, chunk
@@ -88,6 +91,7 @@ struct GemmT96Geometry {
     return 16 * (in_q / 64) + in_q % 16;
   }
 };
+using GemmT96Geometry = GemmT96Tile<96, 96>;
 
 // ---- streaming kernel (gemm_f32_stream.h) ----
 struct GemmStreamGeometry {

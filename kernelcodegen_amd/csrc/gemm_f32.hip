@@ -923,30 +923,48 @@ static GemmPlan default_plan(int64_t M, int64_t N, double *cost_out = nullptr) {
   return plan;
 }
 
-// The 96 x 96 tile (gemm_f32_t96.h): K in whole slices, rows 16-byte aligned.
+// The tiles on 16 x 16 x 4 MFMA blocks (gemm_f32_t96.h: 96 x 96 and 96 x 64): K in whole slices,
+// rows 16-byte aligned.
 static bool t96_shape(int64_t M, int64_t N, int64_t K) {
-  using G = GemmT96Geometry;
-  return M > 0 && N > 0 && K > 0 && N % 4 == 0 && K % G::kBK == 0 && K < (1 << 22) && N < (1 << 22) &&
-         M <= 0x7fffffffLL && ((M + G::kBM - 1) / G::kBM) * ((N + G::kBN - 1) / G::kBN) <= 0x7fffffffLL;
+  return M > 0 && N > 0 && K > 0 && N % 4 == 0 && K % 32 == 0 && K < (1 << 22) && N < (1 << 22) &&
+         M <= 0x7fffffffLL && ((M + 63) / 64) * ((N + 63) / 64) <= 0x7fffffffLL;
 }
-// Its cost in the units of tile_cost; negative where the tile is no candidate.  Measured
-// fraction of MFMA peak with the CUs holding R whole rounds of tiles: 0.83 (R = 1: one wave
-// per SIMD), 0.89 (2), 0.935 (4), 0.95 (9 and more), i.e. about 0.96 - 0.13 / R; scaled by
-// 0.94 like the entries of kTileCands (whose 0.91 for 256 x 128 stands for a measured 0.97).
-// Short K is left to the other tiles: this one stores C in 64-byte row segments.
-static double t96_cost(int64_t M, int64_t N, int64_t K) {
-  using G = GemmT96Geometry;
+// Their cost in the units of tile_cost; negative where a tile is no candidate.  Measured
+// fraction of MFMA peak with the CUs holding R whole rounds of tiles, 96 x 96: 0.83 (R = 1: one
+// wave per SIMD), 0.89 (2), 0.935 (4), 0.95 (9 and more), i.e. about 0.96 - 0.13 / R; 96 x 64:
+// 0.78 (1), 0.90 (2), 0.945 (6), about 0.955 - 0.175 / R; scaled by 0.94 like the entries of
+// kTileCands (whose 0.91 for 256 x 128 stands for a measured 0.97).
+// Short K is left to the other tiles: these store C in 64-byte row segments.
+struct T96Cand {
+  int bn;
+  double eff_many, eff_drop;   // fraction of peak = eff_many - eff_drop / R
+};
+static constexpr T96Cand kT96Cands[] = {{96, 0.96, 0.13}, {64, 0.955, 0.175}};
+static double t96_cost(const T96Cand &c, int64_t M, int64_t N, int64_t K) {
   if (!t96_shape(M, N, K) || K < 512) return -1.0;
-  const int64_t tiles = ((M + G::kBM - 1) / G::kBM) * ((N + G::kBN - 1) / G::kBN);
+  const int64_t tiles = ((M + 95) / 96) * ((N + c.bn - 1) / c.bn);
   if (tiles > 4096) return -1.0;
   const double rounds = static_cast<double>((tiles + kNumCu - 1) / kNumCu);
-  return rounds * G::kBM * G::kBN / (0.94 * (0.96 - 0.13 / rounds));
+  return rounds * 96 * c.bn / (0.94 * (c.eff_many - c.eff_drop / rounds));
 }
-// The model is good to a few per cent: the 96-wide tile must win by that much.
+// the cheaper of the two; *bn_out its BLOCK_SIZE_N
+static double t96_cost(int64_t M, int64_t N, int64_t K, int *bn_out = nullptr) {
+  double best = -1.0;
+  for (const T96Cand &c : kT96Cands) {
+    const double cost = t96_cost(c, M, N, K);
+    if (cost > 0.0 && (best < 0.0 || cost < best)) {
+      best = cost;
+      if (bn_out) *bn_out = c.bn;
+    }
+  }
+  return best;
+}
+// The model is good to a few per cent: a 96-wide tile must win by that much.
 constexpr double kT96Margin = 0.97;
+template <int BM, int BN>
 static int launch_t96(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int epilogue,
                       int group_m, hipStream_t stream, kcg_launch_info *info) {
-  using G = GemmT96Geometry;
+  using G = GemmT96Tile<BM, BN>;
   if (!t96_shape(M, N, K) || !aligned16(A) || !aligned16(B)) return KCG_ERR_BAD_SCHEDULE;
   const int tiles_m = static_cast<int>((M + G::kBM - 1) / G::kBM), tiles_n = static_cast<int>((N + G::kBN - 1) / G::kBN);
   const bool ragged = M % G::kBM != 0 || N % G::kBN != 0;
@@ -960,7 +978,7 @@ static int launch_t96(const float *A, const float *B, float *C, int64_t M, int64
     info->block[1] = info->block[2] = 1;
     info->lds_bytes = G::kLdsBytes;
     info->waves_per_block = G::kWavesM * G::kWavesN;
-    snprintf(info->kernel, sizeof info->kernel, "gemm_f32_96x96x32_w2x2_dl%s", ragged ? "_ragged" : "");
+    snprintf(info->kernel, sizeof info->kernel, "gemm_f32_%dx%dx32_w2x2_dl%s", BM, BN, ragged ? "_ragged" : "");
     return KCG_OK;
   }
   const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n)), block(G::kThreads);
@@ -970,8 +988,8 @@ static int launch_t96(const float *A, const float *B, float *C, int64_t M, int64
                   static_cast<int>(K), tiles_m, tiles_n, group_m);
   };
   const bool relu = epilogue == KCG_EPILOGUE_RELU;
-  if (ragged) return relu ? go(gemm_f32_t96_kernel<true, true>) : go(gemm_f32_t96_kernel<false, true>);
-  return relu ? go(gemm_f32_t96_kernel<true, false>) : go(gemm_f32_t96_kernel<false, false>);
+  if (ragged) return relu ? go(gemm_f32_t96_kernel<BM, BN, true, true>) : go(gemm_f32_t96_kernel<BM, BN, false, true>);
+  return relu ? go(gemm_f32_t96_kernel<BM, BN, true, false>) : go(gemm_f32_t96_kernel<BM, BN, false, false>);
 }
 
 // Resolves a schedule (NULL / zero fields = defaults) to one of the built tile
@@ -985,9 +1003,11 @@ static int launch_sched(const kcg_gemm_sched &d, const float *A, const float *B,
       d.wave_n == BN / WN)                                                                        \
     return launch_gemm<BM, BN, BK, WM, WN, MINW>(A, B, C, M, N, K, epilogue, d.group_m,           \
                                                   d.lds_stages, stream, info);
-  if (d.block_m == 96 && d.block_n == 96 && d.block_k == 32 && d.wave_m == 48 && d.wave_n == 48) {
+  if (d.block_m == 96 && (d.block_n == 96 || d.block_n == 64) && d.block_k == 32 && d.wave_m == 48 &&
+      d.wave_n == d.block_n / 2) {
     if (d.lds_stages == 2) return KCG_ERR_BAD_SCHEDULE;   // built as the direct-load ring only
-    return launch_t96(A, B, C, M, N, K, epilogue, d.group_m, stream, info);
+    return d.block_n == 96 ? launch_t96<96, 96>(A, B, C, M, N, K, epilogue, d.group_m, stream, info)
+                           : launch_t96<96, 64>(A, B, C, M, N, K, epilogue, d.group_m, stream, info);
   }
   KCG_TRY(128, 128, 32, 2, 2, 2)
   KCG_TRY(128, 128, 16, 2, 2, 2)
@@ -1012,11 +1032,14 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
     const bool free_choice = !s || (s->block_k == 0 && s->wave_m == 0 && s->wave_n == 0 && s->lds_stages == 0);
     if (!free_choice) d = default_tile(M, N, 1);
     // extents that 96 divides, where that tile fills the rounds of the CUs better
-    const double c96 = t96_cost(M, N, K);
+    int bn96 = 96;
+    const double c96 = t96_cost(M, N, K, &bn96);
     if (free_choice && c96 > 0.0 && c96 < kT96Margin * plan_cost && aligned16(A) && aligned16(B) &&
         (!s || ((s->wave_size == 0 || s->wave_size == 64) && (s->vec_width == 0 || s->vec_width == 4)))) {
       if (s && s->group_m < 0) return KCG_ERR_BAD_SCHEDULE;
-      return launch_t96(A, B, C, M, N, K, epilogue, s && s->group_m ? s->group_m : 8, stream, info);
+      const int gm = s && s->group_m ? s->group_m : 8;
+      return bn96 == 96 ? launch_t96<96, 96>(A, B, C, M, N, K, epilogue, gm, stream, info)
+                        : launch_t96<96, 64>(A, B, C, M, N, K, epilogue, gm, stream, info);
     }
     if (free_choice && plan.main_rows < M) {
       // caller's remaining fields (GROUP_SIZE_M) apply to both launches

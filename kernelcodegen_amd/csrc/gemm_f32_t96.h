@@ -1,12 +1,12 @@
-// fp32 matmul on a 96 x 96 tile: the tile for problems whose count of such tiles fills the
-// 256 CUs in whole rounds where the power-of-two tiles do not (1536^3 is 256 tiles of
-// 96 x 96, but 576 = 2.25 x 256 tiles of 64 x 64).
+// fp32 matmul on a 96 x 96 or 96 x 64 tile: the tiles for problems whose count of such tiles
+// fills the 256 CUs in whole rounds where the power-of-two tiles do not (1536^3 is 256 tiles
+// of 96 x 96, but 576 = 2.25 x 256 tiles of 64 x 64; 1152^2 is 216 tiles of 96 x 64).
 //
 // Same schedule as gemm_f32_dl_kernel (MatmulOptimizer's, src/Optimizer/Optimizer.cc:383-548:
 // a tile of C per workgroup, K in BLOCK_SIZE_K slices through a ring of LDS stages, later
 // slices in flight during compute, one barrier per slice); what differs is the wave tile.  96
-// is not a multiple of 32 x 2 waves, so the four waves own 48 x 48 each as 3 x 3 blocks of
-// v_mfma_f32_16x16x4_f32 (lane l, r = l % 16, g = l / 16):
+// is not a multiple of 32 x 2 waves, so the four waves own 48 x 48 (or 48 x 32) each as 3 x 3
+// (3 x 2) blocks of v_mfma_f32_16x16x4_f32 (lane l, r = l % 16, g = l / 16):
 //   A operand: A[row r][k = g]      B operand: B[k = g][col r]
 //   D: 4 floats, element e is C[4 * g + e][r].
 // One ds_read_b128 of A gives lane (r, g) the four k = 4g .. 4g+3 of a 16-wide half of the
@@ -26,11 +26,12 @@
 
 namespace kcg {
 
-template <bool RELU, bool RAGGED>
-__global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_kernel(
+template <int BM, int BN, bool RELU, bool RAGGED>
+__global__ __launch_bounds__(256, 2) void gemm_f32_t96_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N, int K,
     int tiles_m, int tiles_n, int group_m) {
-  using G = GemmT96Geometry;
+  using G = GemmT96Tile<BM, BN>;
+  static_assert(G::kThreads == 256, "launch bounds");
   extern __shared__ __align__(16) float lds[];
 
   const int logical = xcd_contiguous_id(blockIdx.x, tiles_m * tiles_n);
@@ -50,11 +51,11 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
   const int r16 = lane & 15;
   const int g = lane >> 4;
 
-  float4_t acc[G::kBlocks][G::kBlocks];
+  float4_t acc[G::kBlocksM][G::kBlocksN];
 #pragma unroll
-  for (int i = 0; i < G::kBlocks; ++i)
+  for (int i = 0; i < G::kBlocksM; ++i)
 #pragma unroll
-    for (int n = 0; n < G::kBlocks; ++n) acc[i][n] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int n = 0; n < G::kBlocksN; ++n) acc[i][n] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   // ---- direct loads: uniform slice base + per-lane 32-bit byte offsets ----
   const int lds_base = static_cast<int>(reinterpret_cast<uintptr_t>(lds));
@@ -106,29 +107,29 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
     for (int h = 0; h < 2; ++h)
       a_addr[st][h] = lds_base + (st * G::kStageFloats + (wm * G::kWaveM + r16) * G::kBK +
                                   4 * ((g + 4 * h) ^ G::fa(r16))) * 4;
-    b_addr[st] = lds_base + (st * G::kStageFloats + G::kFloatsA + wn * G::kBlocks * 64 + g * 16 + r16) * 4;
+    b_addr[st] = lds_base + (st * G::kStageFloats + G::kFloatsA + wn * G::kBlocksN * 64 + g * 16 + r16) * 4;
   }
   static_assert(G::fa(16) == G::fa(0) && G::kWaveM % 16 == 0, "the swizzle repeats every 16 rows");
-  float4_t fa[2][G::kBlocks];
-  float fb[2][G::kBlocks];
-  float4_t na[G::kBlocks];
-  float nb[G::kBlocks];
-  auto read_a = [&](int stage, int h, float4_t(&dst)[G::kBlocks]) {
+  float4_t fa[2][G::kBlocksM];
+  float fb[2][G::kBlocksN];
+  float4_t na[G::kBlocksM];
+  float nb[G::kBlocksN];
+  auto read_a = [&](int stage, int h, float4_t(&dst)[G::kBlocksM]) {
     const int addr = a_addr[stage][h];
 #pragma unroll
-    for (int i = 0; i < G::kBlocks; ++i)
+    for (int i = 0; i < G::kBlocksM; ++i)
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst[i]) : "v"(addr), "n"(i * 16 * G::kBK * 4) : "memory");
   };
-  auto read_b = [&](int stage, int s, float(&dst)[G::kBlocks]) {
+  auto read_b = [&](int stage, int s, float(&dst)[G::kBlocksN]) {
     const int addr = b_addr[stage];
 #pragma unroll
-    for (int n = 0; n < G::kBlocks; ++n)
+    for (int n = 0; n < G::kBlocksN; ++n)
       asm volatile("ds_read_b32 %0, %1 offset:%2"
                    : "=v"(dst[n])
                    : "v"(addr), "n"((s * G::kQuartetFloats + n * 64) * 4)
                    : "memory");
   };
-  constexpr int kReads = G::kBlocks;  // LDS instructions per read_a / read_b
+  constexpr int kReadsA = G::kBlocksM, kReadsB = G::kBlocksN;  // LDS instructions per read_a / read_b
 
   // Publishes the slice requested before the newest one (see gemm_f32_dl_kernel).
   auto publish = [&]() {
@@ -154,9 +155,9 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
   auto drain_reads = [&]() {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < G::kBlocks; ++i) asm volatile("" : "+v"(na[i]));
+    for (int i = 0; i < G::kBlocksM; ++i) asm volatile("" : "+v"(na[i]));
 #pragma unroll
-    for (int n = 0; n < G::kBlocks; ++n) asm volatile("" : "+v"(nb[n]));
+    for (int n = 0; n < G::kBlocksN; ++n) asm volatile("" : "+v"(nb[n]));
   };
   if (first_stage == 0) {
     read_a(0, 0, na);
@@ -178,9 +179,9 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
     constexpr int ST2 = (ST + 2) % G::kStages;
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < G::kBlocks; ++i) fa[0][i] = na[i];
+    for (int i = 0; i < G::kBlocksM; ++i) fa[0][i] = na[i];
 #pragma unroll
-    for (int n = 0; n < G::kBlocks; ++n) fb[0][n] = nb[n];
+    for (int n = 0; n < G::kBlocksN; ++n) fb[0][n] = nb[n];
 #pragma unroll
     for (int s = 0; s < G::kSteps; ++s) {
       // the loads of slice kt+2, one per step
@@ -192,8 +193,8 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
         if (with_a) read_a(ST, (s + 1) / 4, fa[((s + 1) / 4) & 1]);
         read_b(ST, s + 1, fb[(s + 1) & 1]);
         // the operands of step s were requested a step ago: all but this step's reads
-        if (with_a) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(2 * kReads) : "memory");
-        else asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReads) : "memory");
+        if (with_a) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsA + kReadsB) : "memory");
+        else asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsB) : "memory");
       } else {
         publish();  // includes lgkmcnt(0)
         read_a(ST1, 0, na);
@@ -201,9 +202,9 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < G::kBlocks; ++i)
+      for (int i = 0; i < G::kBlocksM; ++i)
 #pragma unroll
-        for (int n = 0; n < G::kBlocks; ++n)
+        for (int n = 0; n < G::kBlocksN; ++n)
           acc[i][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[(s / 4) & 1][i][s % 4], fb[s & 1][n], acc[i][n], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -230,9 +231,9 @@ __global__ __launch_bounds__(GemmT96Geometry::kThreads, 2) void gemm_f32_t96_ker
   const int row0 = m0 + wm * G::kWaveM + 4 * g, col0 = n0 + wn * G::kWaveN + r16;
   float *c_lane = C + static_cast<int64_t>(row0) * N + col0;
 #pragma unroll
-  for (int i = 0; i < G::kBlocks; ++i)
+  for (int i = 0; i < G::kBlocksM; ++i)
 #pragma unroll
-    for (int n = 0; n < G::kBlocks; ++n)
+    for (int n = 0; n < G::kBlocksN; ++n)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float v = acc[i][n][e];

@@ -34,7 +34,8 @@ void KernelCodeGenerator::useCandidateTables() {
   };
   matmulConfigs = {mm(256, 128, 16, 64, 64), mm(256, 128, 32, 64, 64), mm(128, 128, 16, 64, 64),
                    mm(128, 128, 32, 64, 64), mm(128, 128, 8, 64, 64),  mm(128, 64, 32, 64, 32),
-                   mm(64, 64, 32, 32, 32),   mm(96, 96, 32, 48, 48)};
+                   mm(64, 64, 32, 32, 32),   mm(96, 96, 32, 48, 48),
+                   mm(96, 64, 32, 48, 32)};
   // fp32 attention is built for Br 128|256 x Bc 32|64 (not 256 x 64 at head dim 128), bf16 for
   // Br 128|256 x Bc 64; candidates a data type has no kernel for are refused at bind time
   // and score FLT_MAX.

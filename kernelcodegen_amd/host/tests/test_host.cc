@@ -875,7 +875,7 @@ static void test_facade_config_search_and_reference_tile() {
   // the gfx950 search space: every candidate is tried once, the cheapest one is kept,
   // and a candidate the evaluator refuses (FLT_MAX) can never win
   generator.useCandidateTables();
-  CHECK(generator.matmulConfigs.size() == 8 && generator.fmhaConfigs.size() == 4);
+  CHECK(generator.matmulConfigs.size() == 9 && generator.fmhaConfigs.size() == 4);
   std::vector<std::string> seen;
   generator.setEvaluator([&](ModuleOp &m) {
     FuncOp f = Analyzer::collectFunctions(m, "Matmul_m")[0];
@@ -886,7 +886,7 @@ static void test_facade_config_search_and_reference_tile() {
     return tile == "128x128x32" ? 0.5f : 1.0f + static_cast<float>(seen.size());
   });
   auto third = generator.bind(generator.optimize(graph));
-  CHECK(seen.size() == 8 && seen.back() == "96x96x32");
+  CHECK(seen.size() == 9 && seen[7] == "96x96x32" && seen.back() == "96x64x32");
   CHECK(third.size() == 1 && third[0].gemmSched.block_m == 128 && third[0].gemmSched.block_k == 32);
   CHECK(generator.bestLatency() == 0.5f);
   // nothing acceptable: the module stays un-scheduled and nothing binds

@@ -8,7 +8,7 @@
 //     of the slice exactly once per (row, col);
 //   * the stores cover the part of the C tile that lies inside C exactly once (M and N need
 //     not divide the tile: lanes beyond an edge load the last valid row / chunk).
-// usage: gemm_t96_address_model M N K GROUP_M   (prints "... N violations")
+// usage: gemm_t96_address_model BLOCK_N M N K GROUP_M   (BLOCK_N 96 or 64; prints "... N violations")
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -16,7 +16,6 @@
 
 #include "gemm_dl_tile.h"
 
-using G = kcg::GemmT96Geometry;
 
 static long violations = 0;
 static void fail(const char *what, long a, long b, long c) {
@@ -29,10 +28,8 @@ static int xcd_contiguous_id(int w, int n) {
   return xcd * per + (xcd < rem ? xcd : rem) + idx;
 }
 
-int main(int argc, char **argv) {
-  if (argc != 5) return 2;
-  const int64_t M = atoll(argv[1]), N = atoll(argv[2]), K = atoll(argv[3]);
-  const int group_m = atoi(argv[4]);
+template <class G>
+static int replay(int64_t M, int64_t N, int64_t K, int group_m) {
   if (N % 4 || K % G::kBK) return 2;
   const int tiles_m = static_cast<int>((M + G::kBM - 1) / G::kBM), tiles_n = static_cast<int>((N + G::kBN - 1) / G::kBN);
   const int grid = tiles_m * tiles_n;
@@ -108,24 +105,24 @@ int main(int argc, char **argv) {
         const int r16 = lane & 15, g = lane >> 4;
         for (int s = 0; s < G::kSteps; ++s) {
           const int h = s / 4, j = s % 4;
-          for (int i = 0; i < G::kBlocks; ++i) {
+          for (int i = 0; i < G::kBlocksM; ++i) {
             // ds_read_b128 at a_addr[h] + i * 16 rows, element j
             const int fo = (wm * G::kWaveM + r16) * G::kBK + 4 * ((g + 4 * h) ^ G::fa(r16)) + i * 16 * G::kBK + j;
             const int want_row = wm * G::kWaveM + i * 16 + r16, want_k = 16 * h + 4 * g + j;
             if (fo < 0 || fo >= G::kFloatsA || a_img[fo] != want_row * G::kBK + want_k)
               fail("A operand", wave, lane, s);
           }
-          for (int n = 0; n < G::kBlocks; ++n) {
+          for (int n = 0; n < G::kBlocksN; ++n) {
             // ds_read_b32 at b_addr + s quartets + n windows
-            const int fo = wn * G::kBlocks * 64 + g * 16 + r16 + s * G::kQuartetFloats + n * 64;
+            const int fo = wn * G::kBlocksN * 64 + g * 16 + r16 + s * G::kQuartetFloats + n * 64;
             const int want_col = wn * G::kWaveN + n * 16 + r16, want_k = 16 * h + 4 * g + j;
             if (fo < 0 || fo >= G::kFloatsB || b_img[fo] != want_k * G::kBN + want_col)
               fail("B operand", wave, lane, s);
           }
         }
         // D of a block: element e of lane (r16, g) is C[4 * g + e][r16]
-        for (int i = 0; i < G::kBlocks; ++i)
-          for (int n = 0; n < G::kBlocks; ++n)
+        for (int i = 0; i < G::kBlocksM; ++i)
+          for (int n = 0; n < G::kBlocksN; ++n)
             for (int e = 0; e < 4; ++e) {
               const int row = wm * G::kWaveM + i * 16 + 4 * g + e, col = wn * G::kWaveN + n * 16 + r16;
               if (m0 + row >= M || n0 + col >= N) continue;   // the kernel's bounds check
@@ -151,8 +148,18 @@ int main(int argc, char **argv) {
   }
   for (int t = 0; t < grid; ++t)
     if (seen_tile[t] != 1) fail("tile computed other than once", t, seen_tile[t], 0);
-  std::printf("gemm_f32_t96 %lldx%lldx%lld group_m %d: %d workgroups, %ld replayed, %ld violations\n",
-              static_cast<long long>(M), static_cast<long long>(N), static_cast<long long>(K), group_m, grid, checked,
-              violations);
+  std::printf("gemm_f32_t96 tile %dx%d, %lldx%lldx%lld group_m %d: %d workgroups, %ld replayed, %ld violations\n", G::kBM,
+              G::kBN, static_cast<long long>(M), static_cast<long long>(N), static_cast<long long>(K), group_m, grid,
+              checked, violations);
   return violations ? 1 : 0;
+}
+
+int main(int argc, char **argv) {
+  if (argc != 6) return 2;
+  const int bn = atoi(argv[1]);
+  const int64_t M = atoll(argv[2]), N = atoll(argv[3]), K = atoll(argv[4]);
+  const int group_m = atoi(argv[5]);
+  if (bn == 96) return replay<kcg::GemmT96Tile<96, 96>>(M, N, K, group_m);
+  if (bn == 64) return replay<kcg::GemmT96Tile<96, 64>>(M, N, K, group_m);
+  return 2;
 }

@@ -101,6 +101,15 @@ def test_launch_geometry_queries():
     # 1472^3: 16 x 16 tiles of 96 x 96 (the last ones partly outside C) are one round as well
     assert L.kcg_gemm_f32_query(1472, 1472, 1472, None, ctypes.byref(info)) == 0
     assert info.kernel == b"gemm_f32_96x96x32_w2x2_dl_ragged" and info.grid[0] == 256
+    # 1152^2 x 2048: 216 tiles of 96 x 64 are one round, nothing else comes close
+    assert L.kcg_gemm_f32_query(1152, 1152, 2048, None, ctypes.byref(info)) == 0
+    assert info.kernel == b"gemm_f32_96x64x32_w2x2_dl" and info.grid[0] == 12 * 18
+    assert info.lds_bytes == 3 * (96 * 32 + 32 * 64) * 4
+    s64 = lib.GemmSched(block_m=96, block_n=64, block_k=32, wave_m=48, wave_n=32)
+    assert L.kcg_gemm_f32_query(100, 100, 64, ctypes.byref(s64), ctypes.byref(info)) == 0
+    assert info.kernel == b"gemm_f32_96x64x32_w2x2_dl_ragged" and info.grid[0] == 2 * 2
+    s64.wave_n = 48
+    assert L.kcg_gemm_f32_query(100, 100, 64, ctypes.byref(s64), ctypes.byref(info)) == 4
     # the tile by name: K in whole slices, N a multiple of 4, direct-load ring only
     s96 = lib.GemmSched(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
     assert L.kcg_gemm_f32_query(960, 192, 64, ctypes.byref(s96), ctypes.byref(info)) == 0

@@ -126,7 +126,7 @@ def test_k_split_launch_numbering_and_addresses(model, shape):
         assert " 0 violations" in r.stdout
 
 
-# ---- the 96 x 96 tile on 16 x 16 x 4 MFMA blocks (gemm_f32_t96_kernel) ----
+# ---- the 96 x 96 and 96 x 64 tiles on 16 x 16 x 4 MFMA blocks (gemm_f32_t96_kernel) ----
 T96_SRC = os.path.join(ROOT, "tests", "gemm_t96_address_model.cc")
 
 
@@ -144,11 +144,12 @@ def t96_model(tmp_path_factory):
                                   (40032, 384, 32768, 8), (192, 3999936, 32, 8), (1, 4, 32, 8), (97, 100, 96, 3),
                                   (1472, 1500, 64, 8), (40000, 388, 32768, 8)],
                          ids=lambda c: "x".join(map(str, c)))
-def test_t96_loads_operands_and_stores(t96_model, case):
+@pytest.mark.parametrize("block_n", [96, 64])
+def test_t96_loads_operands_and_stores(t96_model, case, block_n):
     """The direct loads of a slice fill its A and B stage exactly once from inside the
     tensors; every operand read of every lane fetches the (row, k) / (k, column) its MFMA step
     multiplies, both operands with the same k and every k of the slice once; the stores of
     the four waves cover the part of the C tile inside C exactly once."""
-    r = subprocess.run([t96_model] + [str(v) for v in case], capture_output=True, text=True, timeout=300)
+    r = subprocess.run([t96_model, str(block_n)] + [str(v) for v in case], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stdout + r.stderr
     assert " 0 violations" in r.stdout

@@ -147,6 +147,7 @@ def test_relu_epilogue_special_values(dev):
 
 
 T96 = dict(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
+T96x64 = dict(block_m=96, block_n=64, block_k=32, wave_m=48, wave_n=32)
 
 
 # K of 1, 2, 3, 5, 48 and 124 slices: every phase of the three-stage ring (K / 32 mod 3 = 1, 2, 0)
@@ -154,16 +155,18 @@ T96 = dict(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
 @pytest.mark.parametrize("shape", [(96, 96, 32), (96, 192, 64), (288, 96, 96), (480, 672, 160), (1536, 1536, 1536),
                                    (960, 1152, 3968), (1, 4, 32), (97, 100, 96), (200, 96, 64), (192, 260, 128),
                                    (1472, 1472, 1472), (1000, 1500, 544)])
-def test_tile_96(oracle, dev, shape):
-    """The 96 x 96 x 32 tile (four waves of 48 x 48 on 16 x 16 x 4 MFMA blocks) by name."""
+@pytest.mark.parametrize("sched", [T96, T96x64], ids=["96x96", "96x64"])
+def test_tile_96(oracle, dev, shape, sched):
+    """The 96 x 96 x 32 and 96 x 64 x 32 tiles (four waves of 48 x 48 / 48 x 32 on 16 x 16 x 4
+    MFMA blocks) by name."""
     from kernelcodegen_amd import ops
     M, N, K = shape
     A = inputs.uniform((M, K), 111, 0)
     B = inputs.uniform((K, N), 111, 1)
     ref = oracle.matmul(A, B)
-    C = ops.matmul(_gpu(A, dev), _gpu(B, dev), sched=T96).cpu().numpy()
+    C = ops.matmul(_gpu(A, dev), _gpu(B, dev), sched=sched).cpu().numpy()
     assert max(rel_err(C, ref)) < TOL
-    Cr = ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=True, sched=T96).cpu().numpy()
+    Cr = ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=True, sched=sched).cpu().numpy()
     assert np.array_equal(Cr, oracle.relu(C))
     assert max(rel_err(Cr, oracle.relu(ref))) < TOL
 
@@ -178,20 +181,23 @@ def test_tile_96_closed_forms_and_default_choice(dev):
     Bi = rng.integers(-8, 9, (512, 384)).astype(np.float32)
     expect = (Ai.astype(np.int64) @ Bi.astype(np.int64)).astype(np.float32)
     assert np.array_equal(ops.matmul(_gpu(Ai, dev), _gpu(Bi, dev), sched=T96).cpu().numpy(), expect)
+    assert np.array_equal(ops.matmul(_gpu(Ai, dev), _gpu(Bi, dev), sched=T96x64).cpu().numpy(), expect)
     # lane mapping of rows, columns and k: A[i,k] = i with B = e_k0 (row k0 of ones) gives C[i,j] = i
     # for every k0 of a slice; A = ones with B[k,j] = j * [k == k0] gives C[i,j] = j
     Am = np.repeat(np.arange(192, dtype=np.float32)[:, None], 64, axis=1)
     for k0 in (0, 5, 19, 31, 32 + 14, 63):
         Bm = np.zeros((64, 288), np.float32)
         Bm[k0] = 1
-        got = ops.matmul(_gpu(Am, dev), _gpu(Bm, dev), sched=T96).cpu().numpy()
-        assert np.array_equal(got, np.repeat(np.arange(192, dtype=np.float32)[:, None], 288, axis=1)), k0
+        for t in (T96, T96x64):
+            got = ops.matmul(_gpu(Am, dev), _gpu(Bm, dev), sched=t).cpu().numpy()
+            assert np.array_equal(got, np.repeat(np.arange(192, dtype=np.float32)[:, None], 288, axis=1)), k0
         Bj = np.zeros((64, 288), np.float32)
         Bj[k0] = np.arange(288)
         Ak = np.zeros((192, 64), np.float32)
         Ak[:, k0] = 1          # only k0 may be picked up: any other k of A against row k0 of B is 0
-        got = ops.matmul(_gpu(Ak, dev), _gpu(Bj, dev), sched=T96).cpu().numpy()
-        assert np.array_equal(got, np.repeat(np.arange(288, dtype=np.float32)[None, :], 192, axis=0)), k0
+        for t in (T96, T96x64):
+            got = ops.matmul(_gpu(Ak, dev), _gpu(Bj, dev), sched=t).cpu().numpy()
+            assert np.array_equal(got, np.repeat(np.arange(288, dtype=np.float32)[None, :], 192, axis=0)), k0
     # 1536^3 takes this tile by default (256 tiles on 256 CUs); GROUP_SIZE_M only renumbers them
     info = lib.LaunchInfo()
     import ctypes
