@@ -88,7 +88,10 @@ typedef struct kcg_gemm_sched {
                       * schedule has 2).  2: slices staged through registers into
                       * double-buffered LDS; 3: ring of three filled by direct
                       * global->LDS loads (needs 16-byte aligned rows, K >= block_k);
-                      * 0: the library chooses (3 where the shape allows, else 2). */
+                      * 1: one copy, the staged schedule that precedes pipeline in the
+                      * reference's recipe (two barriers per slice; built for the
+                      * 128x128x8 and 256x128x16 tiles); 0: the library chooses
+                      * (3 where the shape allows, else 2). */
 } kcg_gemm_sched;
 
 /* C[M,N] = epilogue(A[M,K] . B[K,N]); fp32, row-major, contiguous.

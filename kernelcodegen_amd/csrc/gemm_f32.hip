@@ -68,14 +68,20 @@ __device__ __forceinline__ float4_t load4_dword_aligned(const float *p) {
 // no bounds checks are needed and every global access is a dwordx4.  Otherwise
 // tiles inside C still take vector loads for all but the last, partial K slice.
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool FULL, int MIN_WAVES>
+// BUFS: copies of the K-slice tiles in LDS.  2: the pipelined schedule described below.  1: the
+// staged schedule that precedes Rewriter::pipeline in the reference's recipe (one copy of each
+// shared tile: the next slice waits in registers until every wave has finished the current one,
+// two barriers per slice) -- built so that a nest staged that far runs as it is written.
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RELU, bool FULL, int MIN_WAVES, int BUFS = 2>
 __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f32_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
     int K, int tiles_m, int tiles_n, int group_m) {
   using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N>;
+  static_assert(BUFS == 1 || BUFS == 2, "LDS copies");
   extern __shared__ __align__(16) float lds[];
-  float *As = lds;                     // [2][BM][kPitchA]
-  float *Bs = lds + 2 * T::kFloatsA;   // [2][BK][kPitchB]
+  float *As = lds;                        // [BUFS][BM][kPitchA]
+  float *Bs = lds + BUFS * T::kFloatsA;   // [BUFS][BK][kPitchB]
 
   // ---- workgroup -> C tile (XCD-contiguous, then GROUP_SIZE_M swizzle) ----
   const int logical = xcd_contiguous_id(blockIdx.x, tiles_m * tiles_n);
@@ -207,7 +213,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   for (int g = 0; g < kTransfers; ++g) load_one(g, 0);
 #pragma unroll
   for (int g = 0; g < kTransfers; ++g) store_one(g, 0);
-  if (ktiles > 1) {
+  if (BUFS == 2 && ktiles > 1) {
 #pragma unroll
     for (int g = 0; g < kTransfers; ++g) load_one(g, BK);
   }
@@ -219,20 +225,26 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
   for (int n = 0; n < T::kTilesN; ++n) nb[n] = b_base[n * 32];
 
   for (int kt = 0; kt < ktiles; ++kt) {
-    const int cur = kt & 1;
+    const int cur = BUFS == 2 ? (kt & 1) : 0;
     const float *as = a_base + cur * T::kFloatsA;
     const float *bs = b_base + cur * T::kFloatsB;
 #pragma unroll
     for (int i = 0; i < T::kTilesM; ++i) fa[0][i] = na[i];
 #pragma unroll
     for (int n = 0; n < T::kTilesN; ++n) fb[0][n] = nb[n];
-    if (kt + 1 < ktiles) {
+    if (BUFS == 2) {
+      if (kt + 1 < ktiles) {
 #pragma unroll
-      for (int g = 0; g < kTransfers; ++g) store_one(g, cur ^ 1);
-    }
-    if (kt + 2 < ktiles) {
+        for (int g = 0; g < kTransfers; ++g) store_one(g, cur ^ 1);
+      }
+      if (kt + 2 < ktiles) {
 #pragma unroll
-      for (int g = 0; g < kTransfers; ++g) load_one(g, (kt + 2) * BK);
+        for (int g = 0; g < kTransfers; ++g) load_one(g, (kt + 2) * BK);
+      }
+    } else if (kt + 1 < ktiles) {
+      // one copy: the next slice travels to registers while this one is consumed
+#pragma unroll
+      for (int g = 0; g < kTransfers; ++g) load_one(g, (kt + 1) * BK);
     }
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
@@ -247,7 +259,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
 #pragma unroll
         for (int n = 0; n < T::kTilesN; ++n)
           fb[s1 & 1][n] = bs[((s1 / 4) * 8 + s1 % 4) * T::kPitchB + n * 32];
-      } else {
+      } else if (BUFS == 2) {
         __syncthreads();
         if (kt + 1 < ktiles) {
           const float *as1 = a_base + (cur ^ 1) * T::kFloatsA;
@@ -267,6 +279,17 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWaveSize, MIN_WAVES) void gemm_f
           acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[(s / 4) & 1][i][s % 4], fb[s & 1][n],
                                                            acc[i][n], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (BUFS == 1 && kt + 1 < ktiles) {
+      __syncthreads();   // every wave holds its last operands of slice kt
+#pragma unroll
+      for (int g = 0; g < kTransfers; ++g) store_one(g, 0);
+      __syncthreads();   // slice kt+1 is published
+#pragma unroll
+      for (int i = 0; i < T::kTilesM; ++i)
+        na[i] = *reinterpret_cast<const float4_t *>(a_base + i * 32 * T::kPitchA);
+#pragma unroll
+      for (int n = 0; n < T::kTilesN; ++n) nb[n] = b_base[n * 32];
     }
   }
 
@@ -772,10 +795,14 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
   const bool ragged_dl = !full && (K % 4 == 0) && (N % 4 == 0) && K >= BK && aligned16(A) && aligned16(B);
   const bool relu = epilogue == KCG_EPILOGUE_RELU;
   // lds_stages (the schedule's buffer count): 3 = the direct-load ring, 2 = slices staged
-  // through registers into double-buffered LDS, 0 = the ring where the shape allows it
+  // through registers into double-buffered LDS, 1 = the same with one copy of each tile (built
+  // for the two tiles the host layer stages: 128 x 128 x 8 and 256 x 128 x 16), 0 = the ring
+  // where the shape allows it
+  constexpr bool kHasSingle = (BM == 128 && BN == 128 && BK == 8) || (BM == 256 && BN == 128 && BK == 16);
   const bool dl_shape = (full || ragged_dl) && K < (1 << 22) && N < (1 << 22);
-  const bool use_dl = dl_shape && lds_stages != 2;
+  const bool use_dl = dl_shape && lds_stages != 2 && lds_stages != 1;
   if (lds_stages == 3 && !dl_shape) return KCG_ERR_BAD_SCHEDULE;
+  if (lds_stages == 1 && !kHasSingle) return KCG_ERR_BAD_SCHEDULE;
   if (info) {
     *info = kcg_launch_info{};
     info->launches = 1;
@@ -792,6 +819,10 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
         info->lds_bytes = GemmDlTile<BM, BN, BK, WAVES_M, WAVES_N>::kLdsBytes;
         kind = full ? "_dl" : "_dl_ragged";
       }
+    }
+    if (lds_stages == 1) {
+      info->lds_bytes = T::kLdsBytes / 2;
+      kind = "_single";
     }
     snprintf(info->kernel, sizeof info->kernel, "gemm_f32_%dx%dx%d_w%dx%d%s", BM, BN, BK, WAVES_M,
              WAVES_N, kind);
@@ -814,6 +845,20 @@ static int launch_gemm(const float *A, const float *B, float *C, int64_t M, int6
                     : launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, false, MIN_WAVES>);
       return relu ? launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, true, true, MIN_WAVES>)
                   : launch_dl(gemm_f32_dl_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, true, MIN_WAVES>);
+    }
+  }
+  if constexpr (kHasSingle) {
+    if (lds_stages == 1) {
+      auto launch_single = [&](auto kern) {
+        if (!allow_lds(kern, T::kLdsBytes / 2)) return static_cast<int>(KCG_ERR_LAUNCH);
+        return launch(kern, grid, block, T::kLdsBytes / 2, stream, A, B, C, static_cast<int>(M), static_cast<int>(N),
+                      static_cast<int>(K), static_cast<int>(tiles_m), static_cast<int>(tiles_n), group_m);
+      };
+      if (relu)
+        return full ? launch_single(gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N, true, true, MIN_WAVES, 1>)
+                    : launch_single(gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N, true, false, MIN_WAVES, 1>);
+      return full ? launch_single(gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, true, MIN_WAVES, 1>)
+                  : launch_single(gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N, false, false, MIN_WAVES, 1>);
     }
   }
 #define KCG_LAUNCH(RELU_, FULL_)                                                                 \
@@ -997,7 +1042,7 @@ static int launch_t96(const float *A, const float *B, float *C, int64_t M, int64
 static int launch_sched(const kcg_gemm_sched &d, const float *A, const float *B, float *C, int64_t M, int64_t N,
                         int64_t K, int epilogue, hipStream_t stream, kcg_launch_info *info) {
   if (d.wave_size != 64 || d.vec_width != 4 || d.group_m < 1) return KCG_ERR_BAD_SCHEDULE;
-  if (d.lds_stages != 0 && d.lds_stages != 2 && d.lds_stages != 3) return KCG_ERR_BAD_SCHEDULE;
+  if (d.lds_stages < 0 || d.lds_stages > 3) return KCG_ERR_BAD_SCHEDULE;
 #define KCG_TRY(BM, BN, BK, WM, WN, MINW)                                                         \
   if (d.block_m == BM && d.block_n == BN && d.block_k == BK && d.wave_m == BM / WM &&             \
       d.wave_n == BN / WN)                                                                        \
@@ -1005,7 +1050,7 @@ static int launch_sched(const kcg_gemm_sched &d, const float *A, const float *B,
                                                   d.lds_stages, stream, info);
   if (d.block_m == 96 && (d.block_n == 96 || d.block_n == 64) && d.block_k == 32 && d.wave_m == 48 &&
       d.wave_n == d.block_n / 2) {
-    if (d.lds_stages == 2) return KCG_ERR_BAD_SCHEDULE;   // built as the direct-load ring only
+    if (d.lds_stages == 1 || d.lds_stages == 2) return KCG_ERR_BAD_SCHEDULE;   // built as the direct-load ring only
     return d.block_n == 96 ? launch_t96<96, 96>(A, B, C, M, N, K, epilogue, d.group_m, stream, info)
                            : launch_t96<96, 64>(A, B, C, M, N, K, epilogue, d.group_m, stream, info);
   }

@@ -127,14 +127,8 @@ bool bindMatmul(FuncOp f, KernelBinding &b) {
     b.scheduleSource = "ir";
     b.gemmSched.block_k = static_cast<int>(nest.bk);
     if (nest.vec) b.gemmSched.vec_width = nest.vec;
-    if (nest.copies == 1) {
-      // a single-buffered schedule: the library's least-buffered kernel holds two copies
-      b.gemmSched.lds_stages = 2;
-      b.scheduleNote = "the nest keeps one copy of each shared tile; run on the double-buffered kernel "
-                       "(the library builds no single-buffered one)";
-    } else {
-      b.gemmSched.lds_stages = static_cast<int>(nest.copies);
-    }
+    // one copy of each shared tile (the staged schedule), two (Rewriter::pipeline) or a ring of three
+    b.gemmSched.lds_stages = static_cast<int>(nest.copies);
   }
   const int st = kcg_gemm_f32_query(b.M, b.N, b.K, &b.gemmSched, &b.launch);
   if (st != KCG_OK) {

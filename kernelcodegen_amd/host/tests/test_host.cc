@@ -771,16 +771,16 @@ static void test_schedule_drives_binding() {
       CHECK(contains(src, "from the kcg.* attributes"));
     }
   }
-  {  // staged: one copy of each shared tile -> the double-buffered kernel, with a note
+  {  // staged: one copy of each shared tile -> the single-buffered kernel
     auto [b, src] = bindWith(1);
     CHECK(b.size() == 1);
     if (b.size() == 1) {
       CHECK(b[0].scheduleSource == "ir" && b[0].gemmSched.block_k == 8 && b[0].gemmSched.vec_width == 4);
-      CHECK(b[0].gemmSched.lds_stages == 2 && !b[0].scheduleNote.empty());
-      CHECK(std::string(b[0].launch.kernel) == "gemm_f32_128x128x8_w2x2");
-      CHECK(b[0].launch.lds_bytes == 2 * (128 * (8 + 4) + 8 * (128 + 8)) * 4);
-      CHECK(contains(src, "lds stages 2") && contains(src, "from the scheduled loop nest") && contains(src, "// note: "));
-      CHECK(contains(src, "sched = {128, 128, 8, 8, 64, 64, 4, 64, 2};"));
+      CHECK(b[0].gemmSched.lds_stages == 1 && b[0].scheduleNote.empty());
+      CHECK(std::string(b[0].launch.kernel) == "gemm_f32_128x128x8_w2x2_single");
+      CHECK(b[0].launch.lds_bytes == (128 * (8 + 4) + 8 * (128 + 8)) * 4);
+      CHECK(contains(src, "lds stages 1") && contains(src, "from the scheduled loop nest") && !contains(src, "// note: "));
+      CHECK(contains(src, "sched = {128, 128, 8, 8, 64, 64, 4, 64, 1};"));
     }
   }
   ir::ModuleOp pipelined;
@@ -844,8 +844,11 @@ static void test_schedule_drives_binding() {
     kcg_launch_info info;
     kcg_gemm_sched s = {128, 128, 8, 8, 64, 64, 4, 64, 4};
     CHECK(kcg_gemm_f32_query(512, 384, 256, &s, &info) == KCG_ERR_BAD_SCHEDULE);
-    s.lds_stages = 1;
+    s.lds_stages = 1;   // one copy: built for this tile, not for 128 x 128 x 32
+    CHECK(kcg_gemm_f32_query(512, 384, 256, &s, &info) == KCG_OK && contains(info.kernel, "_single"));
+    s.block_k = 32;
     CHECK(kcg_gemm_f32_query(512, 384, 256, &s, &info) == KCG_ERR_BAD_SCHEDULE);
+    s.block_k = 8;
     s.lds_stages = 3;
     CHECK(kcg_gemm_f32_query(512, 384, 256, &s, &info) == KCG_OK && contains(info.kernel, "_dl"));
     CHECK(kcg_gemm_f32_query(512, 384, 250, &s, &info) == KCG_ERR_BAD_SCHEDULE);  // rows not 16-byte aligned

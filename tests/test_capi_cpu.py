@@ -84,6 +84,16 @@ def test_launch_geometry_queries():
     assert L.kcg_gemm_f32_query(7168, 7168, 7168, None, ctypes.byref(info)) == 0
     assert info.grid[0] == 27 * 56 and info.block[0] == 512
     assert info.kernel == b"gemm_f32_256x128x16_w4x2_dl+256rows_64x64x32"
+    # one copy of the K-slice tiles in LDS: the two tiles the host layer stages, nothing else
+    s1 = lib.GemmSched(block_m=128, block_n=128, block_k=8, wave_m=64, wave_n=64, lds_stages=1)
+    assert L.kcg_gemm_f32_query(4096, 2048, 1024, ctypes.byref(s1), ctypes.byref(info)) == 0
+    assert info.kernel == b"gemm_f32_128x128x8_w2x2_single" and info.lds_bytes == (128 * 12 + 8 * 136) * 4
+    s1.block_k = 16
+    assert L.kcg_gemm_f32_query(4096, 2048, 1024, ctypes.byref(s1), ctypes.byref(info)) == 4
+    s1.block_k, s1.lds_stages = 8, 4
+    assert L.kcg_gemm_f32_query(4096, 2048, 1024, ctypes.byref(s1), ctypes.byref(info)) == 4
+    s1.lds_stages = -1
+    assert L.kcg_gemm_f32_query(4096, 2048, 1024, ctypes.byref(s1), ctypes.byref(info)) == 4
     # an explicit tile is never cut
     s = lib.GemmSched(block_m=256, block_n=128, block_k=16, wave_m=64, wave_n=64)
     assert L.kcg_gemm_f32_query(7168, 7168, 7168, ctypes.byref(s), ctypes.byref(info)) == 0

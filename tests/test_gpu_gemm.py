@@ -146,6 +146,35 @@ def test_relu_epilogue_special_values(dev):
     assert C[4, 9] == 0 and C[5, 10] == np.inf and np.isnan(C[6, 11])
 
 
+@pytest.mark.parametrize("tile", [(128, 128, 8), (256, 128, 16)])
+@pytest.mark.parametrize("shape", [(512, 384, 256), (300, 260, 72), (256, 128, 16), (1024, 1024, 40)])
+def test_lds_buffer_counts(oracle, dev, tile, shape):
+    """kcg_gemm_sched.lds_stages: one copy of the K-slice tiles (the staged schedule), two (the
+    reference's pipeline) and the direct-load ring of three, on the two tiles built for all of
+    them.  One and two copies run the same arithmetic in the same order: bit-identical."""
+    import torch
+    from kernelcodegen_amd import ops
+    from kernelcodegen_amd.lib import KcgError
+    M, N, K = shape
+    bm, bn, bk = tile
+    A = inputs.uniform((M, K), 131, 0)
+    B = inputs.uniform((K, N), 131, 1)
+    ref = oracle.relu(oracle.matmul(A, B))
+    got = {}
+    for stages in (1, 2, 3):
+        sched = dict(block_m=bm, block_n=bn, block_k=bk, wave_m=64, wave_n=64, lds_stages=stages)
+        if stages == 3 and (K % 4 or N % 4 or K < bk):
+            with pytest.raises(KcgError):
+                ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=True, sched=sched)
+            continue
+        got[stages] = ops.matmul(_gpu(A, dev), _gpu(B, dev), relu=True, sched=sched)
+        assert max(rel_err(got[stages].cpu().numpy(), ref)) < TOL, stages
+    assert torch.equal(got[1], got[2])
+    # no single-buffered build of the other tiles
+    with pytest.raises(KcgError):
+        ops.matmul(_gpu(A, dev), _gpu(B, dev), sched=dict(block_m=64, block_n=64, block_k=32, wave_m=32, wave_n=32, lds_stages=1))
+
+
 T96 = dict(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
 T96x64 = dict(block_m=96, block_n=64, block_k=32, wave_m=48, wave_n=32)
 

@@ -38,7 +38,7 @@ def test_matmul_demo(oracle, dev, tmp_path, shape, relu):
     assert max(rel_err(got.reshape(M, N), ref)) < 1e-4
 
 
-@pytest.mark.parametrize("detail,stages,source", [(0, 0, "attributes"), (1, 2, "ir"), (2, 2, "ir"), (3, 3, "ir")])
+@pytest.mark.parametrize("detail,stages,source", [(0, 0, "attributes"), (1, 1, "ir"), (2, 2, "ir"), (3, 3, "ir")])
 @pytest.mark.parametrize("shape", [(512, 384, 256), (384, 640, 72), (300, 260, 72)])
 def test_schedule_selects_the_kernel(oracle, dev, tmp_path, shape, detail, stages, source):
     """The reference's 128 x 128 x 8 tile with the staged (SCHEDULE_DETAIL 1), pipelined (2) and
@@ -59,10 +59,8 @@ def test_schedule_selects_the_kernel(oracle, dev, tmp_path, shape, detail, stage
     assert f[1] == source and int(f[3]) == 8 and int(f[5]) == stages and int(f[7]) == 4
     kernel = f[9]
     assert kernel.startswith("gemm_f32_128x128x8_w2x2")
-    assert ("_dl" in kernel) == (stages != 2)
+    assert ("_dl" in kernel) == (stages in (0, 3)) and kernel.endswith("_single") == (stages == 1)
     assert "static const kcg_gemm_sched sched = {128, 128, 8, 8, 64, 64, 4, 64, %d};" % stages in text
-    if detail == 1 and whole_tiles:
-        assert "// note: the nest keeps one copy of each shared tile" in text
     A = inputs.uniform((M, K), SEED, 0)
     B = inputs.uniform((K, N), SEED, 1)
     ref = oracle.relu(oracle.matmul(A, B))
