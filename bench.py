@@ -14,6 +14,7 @@ depend on how many warm-up steps the caller asks for.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
     python bench.py --sweep matmul [--max-dim D | --dims D1,MxNxK,...] [--relu] [--seeded] [--dump DIR] [--workspace]
+                                   [--series FILE]
     python bench.py --sweep fmha | --sweep ops [--shape B,H,S,D]
     python bench.py --sweep fmha-variants      (after `make -C kernelcodegen_amd/csrc variants`)
 """
@@ -127,6 +128,8 @@ def main():
     ap.add_argument("--relu", action="store_true", help="--sweep matmul: with the fused ReLU epilogue")
     ap.add_argument("--seeded", action="store_true", help="--sweep matmul: operands from the seeded generator")
     ap.add_argument("--dump", help="--sweep matmul: directory that receives sampled rows of every C")
+    ap.add_argument("--series", help="--sweep matmul: JSON file that receives the latency / throughput / peak-ratio "
+                                     "series of the reference's performance/plot.py")
     ap.add_argument("--dims", default="",
                     help="--sweep matmul: comma-separated sizes instead of the reference's list, each n (square) or MxNxK")
     ap.add_argument("--workspace", action="store_true",
@@ -153,7 +156,7 @@ def main():
         if args.sweep == "matmul":
             sweeps.matmul(args.max_dim, args.relu, args.seeded, args.dump, args.workspace,
                           [int(d) if d.isdigit() else tuple(int(x) for x in d.split("x"))
-                           for d in args.dims.split(",")] if args.dims else None)
+                           for d in args.dims.split(",")] if args.dims else None, args.series)
         elif args.sweep == "fmha":
             sweeps.fmha()
         elif args.sweep == "fmha-variants":

@@ -65,7 +65,26 @@ def row_bands(M):
     return [(r0, min(M, r0 + 8)) for r0 in sorted({0, max(0, M // 2 - 4), max(0, M - 8)})]
 
 
-def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=False, dims=None):
+def matmul_series(rows):
+    """The three series the reference's performance/plot.py:43-91 reads out of an output.log
+    (latency, throughput, ratio to peak; one line per method), from rows of (M, N, K, kernel ms,
+    library NN ms, library TT ms).  Throughput is decimal TFLOP/s (plot.py divides by 1024^4 and
+    calls it TFLOPS); the last method is the chip's fp32 matrix peak, as plot.py's is the A100's."""
+    methods = ["Generated-Matmul", "rocm-lib-NN", "rocm-lib-TT", "MI355X-fp32-MFMA-Peak"]
+    dims, latency, throughput, ratio = [], [[] for _ in methods], [[] for _ in methods], [[] for _ in methods]
+    for (M, N, K, mine, nn, tt) in rows:
+        flops = 2.0 * M * N * K
+        dims.append(M if M == N == K else "%dx%dx%d" % (M, N, K))
+        peak_ms = flops / (PEAK_FP32_TFLOPS * 1e9)
+        for i, ms in enumerate((mine, nn, tt, peak_ms)):
+            latency[i].append(ms)
+            throughput[i].append(flops / ms / 1e9)
+            ratio[i].append(100.0 * flops / ms / 1e9 / PEAK_FP32_TFLOPS)
+    return {"methods": methods, "dims": dims, "latency_ms": latency, "throughput_tflops": throughput,
+            "peak_ratio_percent": ratio, "peak_tflops": PEAK_FP32_TFLOPS}
+
+
+def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=False, dims=None, series_path=None):
     import numpy as np
     import torch
     from . import inputs, lib, ops
@@ -75,7 +94,7 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=Fal
     shapes = [(4096, 2048, 1024)] + [(d, d, d) for d in MATMUL_DIMS if d <= max_dim]
     if dims:   # sizes of the caller's choice instead of the reference's list: n (square) or (M, N, K)
         shapes = [(d, d, d) if isinstance(d, int) else tuple(d) for d in dims]
-    rows = []
+    rows, series_rows = [], []
     _settle(dev)
     # --workspace: the calls lend 32 MiB (kcg_gemm_f32_ws), which sizes with a K-split plan use
     ws = torch.empty(8 << 20, dtype=torch.float32, device=dev) if workspace else None
@@ -131,11 +150,16 @@ def matmul(max_dim=16384, relu=False, seeded=False, dump_dir=None, workspace=Fal
         print("rocm-lib Latency(TT) = %g ms\nrocm-lib Ratio(TT) = %g%%\n" % (tt, 100 * tt / mine), flush=True)
         print("max |C - library| / max |C| on sampled rows = %.2g\n" % err, flush=True)
         rows.append((M, N, K, mine, tf, 100 * tf / PEAK_FP32_TFLOPS, nn, flops / nn / 1e9, err))
+        series_rows.append((M, N, K, mine, nn, tt))
         del A, B, C, At, Bt, Ct
     print("| M x N x K | kernel ms | TFLOP/s | % of 157.3 | library NN ms | library TFLOP/s | max err vs library |")
     print("|---|---|---|---|---|---|---|")
     for r in rows:
         print("| %dx%dx%d | %.5g | %.2f | %.1f | %.5g | %.2f | %.1e |" % r)
+    if series_path:
+        import json
+        with open(series_path, "w") as fp:
+            json.dump(matmul_series(series_rows), fp, indent=1)
     return rows
 
 

@@ -27,8 +27,9 @@ BLOCK = re.compile(
 
 @pytest.mark.parametrize("relu", [False, True])
 def test_output_log_fields_and_rows_against_the_oracle(oracle, dev, tmp_path, relu):
+    series_file = os.path.join(str(tmp_path), "series.json")
     cmd = [sys.executable, os.path.join(ROOT, "bench.py"), "--sweep", "matmul", "--max-dim", "1024", "--seeded",
-           "--dump", str(tmp_path)] + (["--relu"] if relu else [])
+           "--dump", str(tmp_path), "--series", series_file] + (["--relu"] if relu else [])
     res = subprocess.run(cmd, capture_output=True, text=True, timeout=600, cwd=ROOT)
     assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
     blocks = BLOCK.findall(res.stdout)
@@ -54,6 +55,18 @@ def test_output_log_fields_and_rows_against_the_oracle(oracle, dev, tmp_path, re
             ref = oracle.relu(ref)
         assert got.shape == ref.shape
         assert max(rel_err(got, ref)) < 1e-4, (M, N, K)
+    # the series performance/plot.py draws (latency, throughput, ratio to peak; four methods)
+    import json
+    with open(series_file) as fp:
+        series = json.load(fp)
+    assert series["dims"] == ["4096x2048x1024", 256, 512, 768, 1024] and len(series["methods"]) == 4
+    for key in ("latency_ms", "throughput_tflops", "peak_ratio_percent"):
+        assert len(series[key]) == 4 and all(len(line) == 5 for line in series[key])
+    for i, b in enumerate(blocks):
+        assert abs(series["latency_ms"][0][i] - float(b[8])) <= 1e-5 * float(b[8]) + 1e-9
+        assert abs(series["latency_ms"][1][i] - float(b[11])) <= 1e-5 * float(b[11]) + 1e-9
+        assert abs(series["throughput_tflops"][0][i] - float(b[9])) < 0.02
+        assert abs(series["peak_ratio_percent"][3][i] - 100.0) < 1e-9
     # the summary table carries one row per size
     assert res.stdout.count("\n| %dx%dx%d |" % want[0]) == 1 and res.stdout.count("\n| 1024x1024x1024 |") == 1
 
