@@ -1065,6 +1065,13 @@ static int launch_sched(const kcg_gemm_sched &d, const float *A, const float *B,
   return KCG_ERR_BAD_SCHEDULE;
 }
 
+// (defined with the BatchedMatmul launchers below)
+static bool stream_shape(int64_t batch, int64_t M, int64_t N, int64_t K, const float *A, const float *B,
+                         const float *C);
+static int launch_bmm_stream(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N,
+                             int64_t K, bool trans_b, bool relu, int group_m, hipStream_t stream,
+                             kcg_launch_info *info);
+
 static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
                          int epilogue, const kcg_gemm_sched *s, hipStream_t stream,
                          kcg_launch_info *info) {
@@ -1076,11 +1083,29 @@ static int dispatch_gemm(const float *A, const float *B, float *C, int64_t M, in
     // a caller who fixes any tile field gets one launch with that field honoured
     const bool free_choice = !s || (s->block_k == 0 && s->wave_m == 0 && s->wave_n == 0 && s->lds_stages == 0);
     if (!free_choice) d = default_tile(M, N, 1);
+    const bool plain_rest = !s || ((s->wave_size == 0 || s->wave_size == 64) && (s->vec_width == 0 || s->vec_width == 4));
+    // A short K (512 to 1024) with at least two whole 256 x 128 tiles per CU: the streaming
+    // kernel of BatchedMatmul, one matrix -- a tile's prologue and its C stores run under the
+    // neighbouring tiles' slices (without an epilogue 8192 x 8192 x 1024: 140 -> 151 TFLOP/s,
+    // 8192 x 4096 x 512: 142 -> 147, 32768 x 768 x 768: 146 -> 148; same tile, slice order and
+    // MFMA mapping: the same bits).  The ReLU epilogue puts two VALU instructions per stored
+    // element into that kernel's slice loop, which costs most of the gain (K = 512: +1 to +4 %,
+    // K = 1024: +-1 %) and more than the gain below K = 512 (-2 % at K = 256): shorter K stays
+    // on the tiled kernel, so that the choice does not depend on the epilogue.
+    // (its workgroups take whole tiles, ceil(tiles / 256) on the busiest CU: only where that
+    // leaves less than 6 % of the last round empty -- the plans below handle the rest better)
+    const int64_t stream_tiles = (M / GemmStreamGeometry::kBM) * (N / GemmStreamGeometry::kBN);
+    const int64_t stream_rounds = (stream_tiles + kNumCu - 1) / kNumCu;
+    if (free_choice && plain_rest && K >= 512 && stream_shape(1, M, N, K, A, B, C) &&
+        stream_tiles * 100 >= stream_rounds * kNumCu * 94) {
+      if (s && s->group_m < 0) return KCG_ERR_BAD_SCHEDULE;
+      return launch_bmm_stream(A, B, C, 1, M, N, K, false, epilogue == KCG_EPILOGUE_RELU, s && s->group_m ? s->group_m : 8,
+                               stream, info);
+    }
     // extents that 96 divides, where that tile fills the rounds of the CUs better
     int bn96 = 96;
     const double c96 = t96_cost(M, N, K, &bn96);
-    if (free_choice && c96 > 0.0 && c96 < kT96Margin * plan_cost && aligned16(A) && aligned16(B) &&
-        (!s || ((s->wave_size == 0 || s->wave_size == 64) && (s->vec_width == 0 || s->vec_width == 4)))) {
+    if (free_choice && c96 > 0.0 && c96 < kT96Margin * plan_cost && aligned16(A) && aligned16(B) && plain_rest) {
       if (s && s->group_m < 0) return KCG_ERR_BAD_SCHEDULE;
       const int gm = s && s->group_m ? s->group_m : 8;
       return bn96 == 96 ? launch_t96<96, 96>(A, B, C, M, N, K, epilogue, gm, stream, info)
@@ -1280,31 +1305,52 @@ static int launch_bmm_dl(const float *A, const float *B, float *C, int64_t batch
 
 // The streaming kernel (gemm_f32_stream.h): one resident workgroup per CU walks its share of
 // the (matrix, tile) list.  Taken when every workgroup has at least two tiles to chain.
+// `relu`: the fused epilogue of the plain matmul (row-major B only).  `info` != nullptr only
+// fills the launch geometry.
 static int launch_bmm_stream(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N,
-                             int64_t K, bool trans_b, hipStream_t stream) {
+                             int64_t K, bool trans_b, bool relu, int group_m, hipStream_t stream,
+                             kcg_launch_info *info) {
+  if (relu && trans_b) return KCG_ERR_BAD_SCHEDULE;
   using G = GemmStreamGeometry;
   const int64_t tiles_m = M / G::kBM, tiles_n = N / G::kBN;
   const int64_t items = tiles_m * tiles_n * batch;
   const int ctas = static_cast<int>(items < kNumCu ? items : kNumCu);
   const bool stream_c = M * N * batch > (int64_t{48} << 20);   // C beyond the last-level cache: non-temporal stores
+  if (info) {
+    *info = kcg_launch_info{};
+    info->launches = 1;
+    info->main_rows = static_cast<int>(M);
+    info->grid[0] = ctas;
+    info->grid[1] = info->grid[2] = 1;
+    info->block[0] = 512;
+    info->block[1] = info->block[2] = 1;
+    info->lds_bytes = G::kStages * GemmDlTile<G::kBM, G::kBN, G::kBK, G::kWavesM, G::kWavesN, false>::kStageFloats * 4;
+    info->waves_per_block = G::kWavesM * G::kWavesN;
+    snprintf(info->kernel, sizeof info->kernel, "gemm_f32_%dx%dx%d_w%dx%d_stream", G::kBM, G::kBN, G::kBK, G::kWavesM,
+             G::kWavesN);
+    return KCG_OK;
+  }
   auto go = [&](auto kern, int lds_bytes) {
     if (!allow_lds(kern, lds_bytes)) return static_cast<int>(KCG_ERR_LAUNCH);
     return launch(kern, dim3(ctas), dim3(512), lds_bytes, stream, A, B, C, static_cast<int>(M), static_cast<int>(N),
-                  static_cast<int>(K), static_cast<int>(tiles_m), static_cast<int>(tiles_n), 8, static_cast<int>(batch),
-                  M * K, K * N, M * N);
+                  static_cast<int>(K), static_cast<int>(tiles_m), static_cast<int>(tiles_n), group_m,
+                  static_cast<int>(batch), M * K, K * N, M * N);
   };
-  auto pick = [&](auto trans_c, auto kt_c) {
+  auto pick = [&](auto trans_c, auto kt_c, auto relu_c) {
     constexpr bool TB = decltype(trans_c)::value;
     constexpr int KT = decltype(kt_c)::value;
+    constexpr bool RL = decltype(relu_c)::value;
     constexpr int lds_bytes =
         G::kStages * GemmDlTile<G::kBM, G::kBN, G::kBK, G::kWavesM, G::kWavesN, TB>::kStageFloats * 4;
-    return stream_c ? go(gemm_f32_stream_kernel<TB, KT, true>, lds_bytes)
-                    : go(gemm_f32_stream_kernel<TB, KT, false>, lds_bytes);
+    return stream_c ? go(gemm_f32_stream_kernel<TB, KT, true, RL>, lds_bytes)
+                    : go(gemm_f32_stream_kernel<TB, KT, false, RL>, lds_bytes);
   };
   using K4 = std::integral_constant<int, 4>;
   using K8 = std::integral_constant<int, 8>;
-  if (trans_b) return K >= 128 ? pick(std::true_type{}, K8{}) : pick(std::true_type{}, K4{});
-  return K >= 128 ? pick(std::false_type{}, K8{}) : pick(std::false_type{}, K4{});
+  using No = std::false_type;
+  if (trans_b) return K >= 128 ? pick(std::true_type{}, K8{}, No{}) : pick(std::true_type{}, K4{}, No{});
+  if (relu) return pick(No{}, K8{}, std::true_type{});   // (the plain matmul only streams from K = 512)
+  return K >= 128 ? pick(No{}, K8{}, No{}) : pick(No{}, K4{}, No{});
 }
 
 static bool stream_shape(int64_t batch, int64_t M, int64_t N, int64_t K, const float *A, const float *B,
@@ -1321,7 +1367,8 @@ static bool stream_shape(int64_t batch, int64_t M, int64_t N, int64_t K, const f
 
 int dispatch_bmm_dl(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N, int64_t K,
                     bool trans_b, hipStream_t stream) {
-  if (stream_shape(batch, M, N, K, A, B, C)) return launch_bmm_stream(A, B, C, batch, M, N, K, trans_b, stream);
+  if (stream_shape(batch, M, N, K, A, B, C))
+    return launch_bmm_stream(A, B, C, batch, M, N, K, trans_b, false, 8, stream, nullptr);
   const kcg_gemm_sched d = default_tile(M, N, batch);
   if (d.block_m == 256) return launch_bmm_dl<256, 128, 16, 4, 2, 2>(A, B, C, batch, M, N, K, trans_b, stream);
   // 128 x 128: the shallow slice has the shorter prologue, which is what counts for the short K

@@ -32,7 +32,7 @@
 
 namespace kcg {
 
-template <bool TRANS_B, int KT, bool STREAM_C>
+template <bool TRANS_B, int KT, bool STREAM_C, bool RELU = false>
 __global__ __launch_bounds__(512, 2) void gemm_f32_stream_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N, int K,
     int tiles_m, int tiles_n, int group_m, int batch, int64_t batch_a, int64_t batch_b, int64_t batch_c) {
@@ -221,7 +221,9 @@ __global__ __launch_bounds__(512, 2) void gemm_f32_stream_kernel(
     constexpr int P = decltype(par_c)::value;
     constexpr int q = decltype(q_c)::value;
     constexpr int i = q / 32, g = (q / 8) % 4, r = (q / 2) % 4, n = q % 2;
-    const float v = acc[P][i][n][4 * g + r];
+    // (RELU, the epilogue of the plain matmul: two VALU instructions per store in the slice
+    // loop, 128 per tile and wave against the tile's K / 2 x 4 MFMAs)
+    const float v = RELU ? relu_maxf(acc[P][i][n][4 * g + r]) : acc[P][i][n][4 * g + r];
     const unsigned off = c_off[i * 4 + g];
     char *const base = c_row[r];
     if (STREAM_C)

@@ -200,10 +200,19 @@ def test_default_matmul_plans_cover_the_problem():
     rng = np.random.default_rng(7)
     shapes = [(d, d) for d in range(1024, 16385, 1024)] + \
              [(int(rng.integers(1, 40000)), int(rng.integers(1, 40000))) for _ in range(300)]
-    cut = 0
+    cut = streamed = 0
     for M, N in shapes:
-        assert L.kcg_gemm_f32_query(M, N, 256, None, ctypes.byref(info)) == 0
+        K = 768 if M == N and M % 1024 == 0 else 256
+        assert L.kcg_gemm_f32_query(M, N, K, None, ctypes.byref(info)) == 0
         name = info.kernel.decode()
+        if name.endswith("_stream"):
+            assert K == 768
+            # a short K (512 to 1024) with whole 256 x 128 tiles, two per CU or more: one persistent
+            # workgroup per CU walks the tiles
+            assert name == "gemm_f32_256x128x16_w4x2_stream" and M % 256 == 0 and N % 128 == 0
+            assert (M // 256) * (N // 128) >= 512 and info.grid[0] == 256 and info.block[0] == 512
+            streamed += 1
+            continue
         m = re.fullmatch(r"gemm_f32_(\d+)x(\d+)x(\d+)_w\dx\d(?:_dl|_dl_ragged)?(?:\+(\d+)rows_(\d+)x(\d+)x(\d+))?", name)
         assert m, name
         bm, bn = int(m.group(1)), int(m.group(2))
@@ -216,7 +225,7 @@ def test_default_matmul_plans_cover_the_problem():
             cut += 1
             assert (bm, bn) == (256, 128) and main_rows + int(m.group(4)) == M, (M, N, name)
             assert int(m.group(4)) >= 1
-    assert cut > 10      # the sweep's odd multiples of 1024 at least
+    assert cut > 10 and streamed >= 5
 
 
 def _meta(shape, dtype, cuda=True, contiguous=True):

@@ -175,6 +175,34 @@ def test_lds_buffer_counts(oracle, dev, tile, shape):
         ops.matmul(_gpu(A, dev), _gpu(B, dev), sched=dict(block_m=64, block_n=64, block_k=32, wave_m=32, wave_n=32, lds_stages=1))
 
 
+@pytest.mark.parametrize("shape", [(4096, 4096, 512), (8192, 2048, 576), (2048, 8192, 1024), (32768, 768, 768)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_short_k_matmul_on_the_streaming_kernel(oracle, dev, shape, relu):
+    """A short K (512 to 1024) with two or more whole 256 x 128 tiles per CU runs on the streaming kernel (one
+    persistent workgroup per CU, the ring of K slices running across tile boundaries, C of a
+    tile stored under the next tile's slices), here with the fused epilogue.  Same tile, slice
+    order and MFMA mapping as the 256 x 128 x 16 direct-load kernel: bit-identical to it."""
+    import ctypes
+    import torch
+    from kernelcodegen_amd import ops, lib
+    M, N, K = shape
+    info = lib.LaunchInfo()
+    assert lib.load().kcg_gemm_f32_query(M, N, K, None, ctypes.byref(info)) == 0
+    assert info.kernel == b"gemm_f32_256x128x16_w4x2_stream" and info.grid[0] == 256
+    A = inputs.uniform((M, K), 141, 0)
+    B = inputs.uniform((K, N), 141, 1)
+    Ag, Bg = _gpu(A, dev), _gpu(B, dev)
+    C = ops.matmul(Ag, Bg, relu=relu)
+    tiled = ops.matmul(Ag, Bg, relu=relu, sched=dict(block_m=256, block_n=128, block_k=16, wave_m=64, wave_n=64))
+    assert torch.equal(C, tiled)
+    # sampled row bands against the oracle (the whole product of the largest shape takes the CPU a while)
+    for r0 in (0, M // 2 - 64, M - 128):
+        ref = oracle.matmul(np.ascontiguousarray(A[r0:r0 + 128]), B)
+        if relu:
+            ref = oracle.relu(ref)
+        assert max(rel_err(C[r0:r0 + 128].cpu().numpy(), ref)) < TOL
+
+
 T96 = dict(block_m=96, block_n=96, block_k=32, wave_m=48, wave_n=48)
 T96x64 = dict(block_m=96, block_n=64, block_k=32, wave_m=48, wave_n=32)
 
