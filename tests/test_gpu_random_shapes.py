@@ -115,3 +115,38 @@ def test_batched_matmul_random_shapes(oracle, dev):
         C = ops.batched_matmul(_gpu(A, dev), _gpu(B, dev), trans_a=ta, trans_b=tb).cpu().numpy()
         assert C.shape == ref.shape
         assert max(rel_err(C, ref)) < 1e-4, (case, batch, M, N, K, ta, tb)
+
+
+def test_repeated_launches_give_the_same_bits(dev):
+    """Every kernel here sums in a fixed order, and operand registers are refilled from LDS
+    behind the MFMAs that read them: a refill that overtook its reader, or any other race,
+    would show as a launch whose bits differ.  Forty launches of each of the main kernels
+    against the first one."""
+    import torch
+    from kernelcodegen_amd import ops
+    g = torch.Generator(device="cpu").manual_seed(77)
+    cases = []
+    A = torch.randn(2048, 1024, generator=g).to(dev)
+    B = torch.randn(1024, 1536, generator=g).to(dev)
+    cases.append(("matmul 256x128 / default", lambda: ops.matmul(A, B, relu=True)))
+    A96 = torch.randn(1536, 1536, generator=g).to(dev)
+    B96 = torch.randn(1536, 1536, generator=g).to(dev)
+    cases.append(("matmul 96x96", lambda: ops.matmul(A96, B96)))
+    cases.append(("matmul 96x64", lambda: ops.matmul(A96[:1152, :1024].contiguous(), B96[:1024, :1152].contiguous())))
+    As = torch.randn(4096, 768, generator=g).to(dev)
+    Bs = torch.randn(768, 4096, generator=g).to(dev)
+    cases.append(("matmul streaming", lambda: ops.matmul(As, Bs)))
+    Q, K, V = (torch.randn(2, 8, 2048, 128, generator=g).to(dev) for _ in range(3))
+    Qb, Kb, Vb = (t.to(torch.bfloat16) for t in (Q, K, V))
+    Qs, Ks, Vs = (t[:, :, :1024].contiguous() for t in (Q, K, V))
+    for causal in (False, True):
+        cases.append(("fmha f32 causal=%d" % causal, lambda c=causal: ops.fmha(Qs, Ks, Vs, scale=0.088, causal=c)))
+        cases.append(("fmha bf16 ping-pong causal=%d" % causal,
+                      lambda c=causal: ops.fmha(Qb, Kb, Vb, scale=0.088, causal=c, sched=dict(br=256, bc=64))))
+        cases.append(("fmha bf16 128-row causal=%d" % causal,
+                      lambda c=causal: ops.fmha(Qb, Kb, Vb, scale=0.088, causal=c, sched=dict(br=128, bc=64))))
+    for name, fn in cases:
+        first = fn()
+        assert bool(torch.isfinite(first.float()).all()), name
+        for _ in range(40):
+            assert torch.equal(fn(), first), name
